@@ -1,0 +1,94 @@
+// Shared helpers of the HIP sources: error reporting, dtype tags, reductions, bf16 conversion.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+enum LevDtype { LEV_F32 = 0, LEV_BF16 = 1 };
+enum LevAct { LEV_ACT_NONE = 0, LEV_ACT_GELU_TANH = 1, LEV_ACT_GELU_ERF = 2, LEV_ACT_RELU = 3, LEV_ACT_SILU = 4,
+              LEV_ACT_QUICK_GELU = 5, LEV_ACT_TANH = 6 };
+
+// ---- errors: every entry point returns 0 or a negative code and leaves a message here
+extern "C" const char* lev_last_error();
+int lev_fail(const char* fmt, ...);
+int lev_check_launch(const char* what);
+
+#define LEV_REQUIRE(cond, ...)            \
+  do {                                    \
+    if (!(cond)) return lev_fail(__VA_ARGS__); \
+  } while (0)
+
+// ---- bf16 as raw 16 bits -----------------------------------------------------------------
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_float(T v);
+template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return bf16_to_float(v); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
+
+// ---- wave (64 lanes) and block reductions ---------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// sum over a block of NT threads (NT a multiple of 64, at most 1024); every thread gets the result.
+// `red` is shared memory of at least NT/64 floats. Safe to call repeatedly (syncs before reuse).
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  if (NT == 64) return v;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) t += red[i];
+  return t;
+}
+template <int NT> __device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  if (NT == 64) return v;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int i = 1; i < NT / 64; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+// ---- activation functions, in 32-bit --------------------------------------------------------
+__device__ __forceinline__ float lev_activate(float u, int act) {
+  switch (act) {
+    case LEV_ACT_GELU_TANH: {
+      const float c = 0.7978845608028654f;  // sqrt(2/pi)
+      return 0.5f * u * (1.0f + tanhf(c * (u + 0.044715f * u * u * u)));
+    }
+    case LEV_ACT_GELU_ERF: return 0.5f * u * (1.0f + erff(u * 0.7071067811865476f));
+    case LEV_ACT_RELU: return fmaxf(u, 0.f);
+    case LEV_ACT_SILU: return u / (1.0f + expf(-u));
+    case LEV_ACT_QUICK_GELU: return u / (1.0f + expf(-1.702f * u));
+    case LEV_ACT_TANH: return tanhf(u);
+    default: return u;
+  }
+}

@@ -1,0 +1,216 @@
+// Embedding gather-add, LayerNorm / RMSNorm, the write of new keys and values into pages, sampling.
+#include "common.h"
+
+// ------------------------------------------------------------------------------------------
+// x[t, :] = float(table[token_t, :]) + float(pos_table[pos_t, :])        (32-bit residual stream)
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                             const T* __restrict__ table, const T* __restrict__ pos_table, float* __restrict__ out, int D) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)tokens[t] * D;
+  const T* prow = pos_table ? pos_table + (size_t)positions[t] * D : nullptr;
+  float* o = out + (size_t)t * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float v = to_float<T>(row[d]);
+    if (prow) v += to_float<T>(prow[d]);
+    o[d] = v;
+  }
+}
+
+extern "C" int lev_embed(const int* tokens, const int* positions, const void* table, const void* pos_table, float* out,
+                         int T, int D, int dtype, hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && D > 0, "embed: bad sizes T=%d D=%d", T, D);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "embed: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  if (dtype == LEV_F32)
+    embed_kernel<float><<<T, 256, 0, stream>>>(tokens, positions, (const float*)table, (const float*)pos_table, out, D);
+  else
+    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(tokens, positions, (const bf16_t*)table, (const bf16_t*)pos_table, out, D);
+  return lev_check_launch("embed");
+}
+
+// ------------------------------------------------------------------------------------------
+// One block per output row. Statistics in 32-bit, two passes (mean, then the centred squares).
+// rows != null: output row r is the norm of input row rows[r] (the wanted rows before the head).
+template <typename TO, int NT>
+__global__ void norm_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b,
+                            TO* __restrict__ out, const int* __restrict__ rows, int D, float eps, int rms) {
+  __shared__ float red[NT / 64];
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * D;
+  float mean = 0.f;
+  if (!rms) {
+    float s = 0.f;
+    for (int d = threadIdx.x; d < D; d += NT) s += xr[d];
+    mean = block_sum<NT>(s, red) / (float)D;
+  }
+  float s2 = 0.f;
+  for (int d = threadIdx.x; d < D; d += NT) {
+    float c = xr[d] - mean;
+    s2 += c * c;
+  }
+  const float var = block_sum<NT>(s2, red) / (float)D;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  TO* o = out + (size_t)r * D;
+  for (int d = threadIdx.x; d < D; d += NT) {
+    float y = (xr[d] - mean) * rstd * w[d];
+    if (b) y += b[d];
+    o[d] = from_float<TO>(y);
+  }
+}
+
+extern "C" int lev_norm(const float* x, const float* w, const float* b, void* out, const int* rows, int n_rows, int D,
+                        float eps, int rms, int out_dtype, hipStream_t stream) {
+  LEV_REQUIRE(n_rows >= 0 && D > 0, "norm: bad sizes rows=%d D=%d", n_rows, D);
+  LEV_REQUIRE(out_dtype == LEV_F32 || out_dtype == LEV_BF16, "norm: unknown output dtype %d", out_dtype);
+  LEV_REQUIRE(eps > 0.f, "norm: eps must be positive");
+  if (n_rows == 0) return 0;
+  if (out_dtype == LEV_F32)
+    norm_kernel<float, 256><<<n_rows, 256, 0, stream>>>(x, w, b, (float*)out, rows, D, eps, rms);
+  else
+    norm_kernel<bf16_t, 256><<<n_rows, 256, 0, stream>>>(x, w, b, (bf16_t*)out, rows, D, eps, rms);
+  return lev_check_launch("norm");
+}
+
+// ------------------------------------------------------------------------------------------
+// New keys and values into their pages. Page layouts (elements):
+//   keys   [page][kv_head][head_dim/8][page_size][8]
+//   values [page][kv_head][head_dim][page_size]
+// dest[t] = page * page_size + offset in page; a negative dest drops the token.
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v, long k_stride, long v_stride,
+                                T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ dest, int KVH,
+                                int HD, int PS) {
+  const int t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int dst = dest[t];
+  if (dst < 0) return;
+  const int page = dst / PS, off = dst % PS;
+  const size_t base = ((size_t)page * KVH + h) * (size_t)HD * PS;
+  const T* kr = k + (size_t)t * k_stride + (size_t)h * HD;
+  const T* vr = v + (size_t)t * v_stride + (size_t)h * HD;
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    k_pages[base + ((size_t)(d >> 3) * PS + off) * 8 + (d & 7)] = kr[d];
+    v_pages[base + (size_t)d * PS + off] = vr[d];
+  }
+}
+
+extern "C" int lev_kv_write(const void* k, const void* v, long k_stride, long v_stride, void* k_pages, void* v_pages,
+                            const int* dest, int T, int KVH, int HD, int PS, int dtype, hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && KVH > 0, "kv_write: bad sizes T=%d kv_heads=%d", T, KVH);
+  LEV_REQUIRE(HD > 0 && HD % 8 == 0, "kv_write: head_dim=%d must be a multiple of 8", HD);
+  LEV_REQUIRE(PS > 0 && PS % 16 == 0, "kv_write: page_size=%d must be a multiple of 16", PS);
+  LEV_REQUIRE(KVH <= 65535, "kv_write: too many kv heads (%d)", KVH);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "kv_write: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  dim3 grid(T, KVH);
+  const int nt = HD <= 64 ? 64 : (HD <= 128 ? 128 : 256);
+  if (dtype == LEV_F32)
+    kv_write_kernel<float><<<grid, nt, 0, stream>>>((const float*)k, (const float*)v, k_stride, v_stride, (float*)k_pages,
+                                                    (float*)v_pages, dest, KVH, HD, PS);
+  else
+    kv_write_kernel<bf16_t><<<grid, nt, 0, stream>>>((const bf16_t*)k, (const bf16_t*)v, k_stride, v_stride,
+                                                     (bf16_t*)k_pages, (bf16_t*)v_pages, dest, KVH, HD, PS);
+  return lev_check_launch("kv_write");
+}
+
+// ------------------------------------------------------------------------------------------
+// Sampling. One block per row of 32-bit logits.
+//   temperature == 0: token = argmax(logits) (ties: the lowest index), logprob from the raw logits;
+//   otherwise: token = argmax(logits / T + Gumbel noise), logprob = (logits/T)[token] - logsumexp(logits/T).
+// The noise of vocabulary entry v comes from Philox4x32-10 with the row's 64-bit key and the counter
+// (v / 4, position, 0, 0), lane v % 4: it depends on (key, position, v) and on nothing else.
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                              uint32_t out[4]) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+__device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
+  const float u = ((float)(bits >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+  return -logf(-logf(u));
+}
+
+struct ArgMax {
+  float v;
+  int i;
+};
+__device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
+template <int NT>
+__global__ void sample_kernel(const float* __restrict__ logits, long row_stride, const float* __restrict__ temperature,
+                              const uint32_t* __restrict__ keys, const int* __restrict__ positions, int* __restrict__ tokens,
+                              float* __restrict__ logprobs, int V) {
+  __shared__ float red[NT / 64];
+  __shared__ float sv[NT / 64];
+  __shared__ int si[NT / 64];
+  const int r = blockIdx.x;
+  const float* lg = logits + (size_t)r * row_stride;
+  const float temp = temperature[r];
+  const bool greedy = (temp == 0.0f);
+  const float safe_t = greedy ? 1.0f : temp;
+  const uint32_t k0 = keys[2 * r], k1 = keys[2 * r + 1];
+  const uint32_t pos = (uint32_t)positions[r];
+
+  ArgMax best = {-INFINITY, 0x7fffffff};
+  float mx = -INFINITY;
+  for (int g = threadIdx.x; g * 4 < V; g += NT) {
+    uint32_t rnd[4] = {0, 0, 0, 0};
+    if (!greedy) philox4x32_10((uint32_t)g, pos, 0u, 0u, k0, k1, rnd);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int v = g * 4 + j;
+      if (v < V) {
+        const float s = lg[v] / safe_t;
+        mx = fmaxf(mx, s);
+        const float c = greedy ? s : s + gumbel_from_bits(rnd[j]);
+        best = better(best, ArgMax{c, v});
+      }
+    }
+  }
+  // block argmax
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ArgMax other = {__shfl_xor(best.v, o, 64), __shfl_xor(best.i, o, 64)};
+    best = better(best, other);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = best.v;
+    si[threadIdx.x >> 6] = best.i;
+  }
+  mx = block_max<NT>(mx, red);  // syncs: sv / si are visible afterwards
+  ArgMax top = {sv[0], si[0]};
+#pragma unroll
+  for (int i = 1; i < NT / 64; ++i) top = better(top, ArgMax{sv[i], si[i]});
+  float se = 0.f;
+  for (int v = threadIdx.x; v < V; v += NT) se += expf(lg[v] / safe_t - mx);
+  se = block_sum<NT>(se, red);
+  if (threadIdx.x == 0) {
+    const int tok = top.i < V ? top.i : 0;
+    tokens[r] = tok;
+    logprobs[r] = lg[tok] / safe_t - mx - logf(se);
+  }
+}
+
+extern "C" int lev_sample(const float* logits, long row_stride, const float* temperature, const uint32_t* keys,
+                          const int* positions, int* tokens, float* logprobs, int R, int V, hipStream_t stream) {
+  LEV_REQUIRE(R >= 0 && V > 0, "sample: bad sizes rows=%d vocab=%d", R, V);
+  LEV_REQUIRE(row_stride >= V, "sample: row stride %ld is smaller than the vocabulary %d", row_stride, V);
+  if (R == 0) return 0;
+  sample_kernel<256><<<R, 256, 0, stream>>>(logits, row_stride, temperature, keys, positions, tokens, logprobs, V);
+  return lev_check_launch("sample");
+}

@@ -1,0 +1,55 @@
+"""From a model folder (or a configuration and a seed) to a runnable model and its runner.
+
+The model class is chosen by ``config.json`` through the registry, as the reference does with
+``config.model_type`` and ``converter.load_pretrained`` (src/levanter/main/sample_lm.py:64-89,
+src/levanter/compat/hf_checkpoints.py:609-701)."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from levanter_amd.cache import CacheManager
+from levanter_amd.config import InferenceEngineConfig, LmConfig
+from levanter_amd.kernels import get_kernels
+from levanter_amd.parts import BuildEnv, DecoderLm
+from levanter_amd.weights import load_tensors, random_tensors
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
+        return dtype
+    try:
+        return DTYPES[str(dtype)]
+    except KeyError:
+        raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype!r}") from None
+
+
+def make_env(dtype, device: Optional[str] = None) -> BuildEnv:
+    """The build environment on the GPU; raises if there is none (no CPU path)."""
+    kernels = get_kernels()
+    dev = torch.device(device or "cuda:0")
+    return BuildEnv(dtype=resolve_dtype(dtype), device=dev, kernels=kernels)
+
+
+def load_model(model_dir: str, env: BuildEnv) -> Tuple[LmConfig, DecoderLm]:
+    config = LmConfig.load(model_dir)
+    spec = config.model_spec()
+    tensors = load_tensors(model_dir, spec, device="cpu")
+    return config, DecoderLm(spec, tensors, env)
+
+
+def random_model(config: LmConfig, seed: int, env: BuildEnv) -> DecoderLm:
+    """A model with random weights drawn on the model's device (no folder is written)."""
+    spec = config.model_spec()
+    tensors = random_tensors(spec, seed, dtype=env.dtype, device=env.device)
+    return DecoderLm(spec, tensors, env)
+
+
+def make_cache(model: DecoderLm, cfg: InferenceEngineConfig) -> CacheManager:
+    return CacheManager(model.cache_requirements(), n_pages=cfg.imputed_max_pages, page_size=cfg.page_size,
+                        max_seqs=cfg.max_seqs, max_pages_per_seq=cfg.max_pages_per_seq)

@@ -1,0 +1,186 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+The reference's counterpart is ``model.decode(tokens, cache, batch_info, pos_ids)``
+(src/levanter/models/llama.py:589-633) fed by ``PageTable.allocate_for_seq`` and
+``PageBatchInfo`` (src/levanter/inference/page_table.py:142-324,508-542): each request
+contributes a contiguous run of tokens whose positions continue its cache, pages are taken
+lazily for the positions the run reaches, every new token gets the destination
+``page * page_size + position % page_size``, and attention sees ``kv_len - q_len`` earlier
+tokens plus the run itself. Here the batch has exactly the tokens it is given (no padding), the
+tables are built on the host and go to the GPU in one copy, and only the wanted rows pass the
+final norm and the head.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from levanter_amd.cache import NO_PAGE, CacheManager, OutOfPages, SequenceHandle
+from levanter_amd.parts.base import AttentionMeta, BuildEnv, CacheUnitView, GroupView, StepContext
+from levanter_amd.parts.decoder import DecoderLm
+
+PREFILL_TILE_ROWS = 64
+
+
+@dataclass
+class StepEntry:
+    """A request's part in a step: its next tokens and the places among them whose logits are wanted."""
+
+    handle: SequenceHandle
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class StepError(ValueError):
+    """A step that cannot run: a bad token id, a position beyond the model's range, a bad ``want``."""
+
+
+class ModelRunner:
+    """Owns the model, the cache manager's device tensors and the step function."""
+
+    def __init__(self, model: DecoderLm, cache: CacheManager, env: BuildEnv, allocate: bool = True):
+        self.model = model
+        self.cache = cache
+        self.env = env
+        if allocate:
+            cache.allocate_tensors(env.dtype, env.device)
+        self._workspaces: Dict[object, torch.Tensor] = {}
+        limit = cache.page_size * cache.max_pages_per_seq
+        mp = model.max_positions
+        self.max_len = limit if mp is None else min(limit, mp)
+
+    # ------------------------------------------------------------------------------------
+    def pages_needed(self, entries: Sequence[StepEntry]) -> List[int]:
+        """Pages each group would have to find for these entries."""
+        return [sum(g.blocks_needed(e.handle.slot, e.handle.length, e.handle.length + len(e.tokens)) for e in entries)
+                for g in self.cache.groups]
+
+    def fits(self, entries: Sequence[StepEntry]) -> bool:
+        return all(n <= g.pool.n_free for n, g in zip(self.pages_needed(entries), self.cache.groups))
+
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        seen = set()
+        v = self.model.vocab_size
+        for e in entries:
+            n = len(e.tokens)
+            rid = e.handle.request_id
+            if e.handle.closed:
+                raise StepError(f"request {rid!r} has ended")
+            if e.handle.slot in seen:
+                raise StepError(f"request {rid!r} appears twice in one step")
+            seen.add(e.handle.slot)
+            if n == 0:
+                raise StepError(f"request {rid!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < v:
+                    raise StepError(f"request {rid!r}: token id {t} is outside the vocabulary of {v}")
+            if e.handle.length + n > self.max_len:
+                raise StepError(f"request {rid!r} would reach {e.handle.length + n} tokens; the limit is {self.max_len} "
+                                f"(positions of the model and page_size * max_pages_per_seq)")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"request {rid!r}: wanted place {w} is not among its {n} tokens")
+
+    # ------------------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries as one batch. Returns float32 logits [wanted, vocab] in the order of the
+        entries and of their ``want``. Raises ``OutOfPages`` (nothing changed) if a pool is too small."""
+        entries = list(entries)
+        self._validate(entries)
+        if not entries:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.env.device)
+        if not self.fits(entries):
+            need = self.pages_needed(entries)
+            raise OutOfPages("out of free pages: the step needs " + ", ".join(
+                f"{n} of group {g.index}'s {g.pool.n_free} free" for n, g in zip(need, self.cache.groups)))
+        for e in entries:
+            self.cache.extend(e.handle, len(e.tokens))
+
+        cache, ps = self.cache, self.cache.page_size
+        S = len(entries)
+        T = sum(len(e.tokens) for e in entries)
+        tokens = np.empty(T, np.int32)
+        positions = np.empty(T, np.int32)
+        token_seq = np.empty(T, np.int32)
+        seq_slots = np.empty(S, np.int32)
+        rows: List[int] = []
+        tiles: List[int] = []
+        decode: List[int] = []
+        run_lengths, first_positions = [], []
+        max_blocks, max_kv = 1, 1
+        t0 = 0
+        for s, e in enumerate(entries):
+            n, start = len(e.tokens), e.handle.length
+            tokens[t0:t0 + n] = np.asarray(e.tokens, dtype=np.int64)
+            positions[t0:t0 + n] = np.arange(start, start + n)
+            token_seq[t0:t0 + n] = s
+            seq_slots[s] = e.handle.slot
+            rows.extend(t0 + int(w) for w in e.want)
+            if n == 1:
+                decode.append(t0)
+            else:
+                for r0 in range(0, n, PREFILL_TILE_ROWS):
+                    tiles.extend((t0 + r0, min(PREFILL_TILE_ROWS, n - r0)))
+            run_lengths.append(n)
+            first_positions.append(start)
+            max_blocks = max(max_blocks, (start + n + ps - 1) // ps)
+            max_kv = max(max_kv, start + n)
+            t0 += n
+
+        n_groups = len(cache.groups)
+        # one int32 buffer for everything that goes to the GPU
+        sizes = [T, T, T, S, len(rows), len(tiles), len(decode)] + [S * max_blocks, T] * n_groups
+        offs = np.concatenate([[0], np.cumsum([(x + 3) // 4 * 4 for x in sizes])]).astype(np.int64)
+        host = np.zeros(int(offs[-1]), np.int32)
+        for i, arr in enumerate((tokens, positions, token_seq, seq_slots, rows, tiles, decode)):
+            host[offs[i]:offs[i] + sizes[i]] = arr
+        for gi, g in enumerate(cache.groups):
+            bt = g.block_tables[seq_slots, :max_blocks]
+            host[offs[7 + 2 * gi]:offs[7 + 2 * gi] + S * max_blocks] = bt.reshape(-1)
+            dest = np.empty(T, np.int32)
+            t0 = 0
+            for s, e in enumerate(entries):
+                n, start = len(e.tokens), e.handle.length
+                pos = np.arange(start, start + n)
+                pages = g.block_tables[e.handle.slot, pos // ps]
+                assert (pages != NO_PAGE).all(), "a new token has no page"
+                dest[t0:t0 + n] = pages * ps + pos % ps
+                t0 += n
+            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = dest
+        dev = self._upload(host)
+
+        def view(i):
+            return dev[int(offs[i]):int(offs[i]) + sizes[i]]
+
+        meta = AttentionMeta(
+            positions=view(1), token_seq=view(2),
+            prefill_tiles=view(5).view(-1, 2) if tiles else None, n_prefill_tiles=len(tiles) // 2,
+            decode_tokens=view(6) if decode else None, n_decode=len(decode),
+            max_kv_len=max_kv, _workspaces=self._workspaces)
+        ctx = StepContext(kernels=self.env.kernels, dtype=self.env.dtype, device=self.env.device, n_tokens=T, tokens=view(0),
+                          attention=meta, seq_slots=view(3),
+                          host={"run_lengths": run_lengths, "first_positions": first_positions,
+                                "slots": [int(s) for s in seq_slots]})
+        group_views = [GroupView(page_size=ps, block_tables=view(7 + 2 * gi).view(S, max_blocks), dest=view(8 + 2 * gi))
+                       for gi in range(n_groups)]
+        for unit, g in cache.group_of_unit.items():
+            i = g.unit_pos[unit]
+            ctx.units[unit] = CacheUnitView(k_pages=g.k_pages[i], v_pages=g.v_pages[i], group=group_views[g.index])
+        for unit, t in cache.state.tensors.items():
+            ctx.units[unit] = CacheUnitView(state=t)
+        for e in self.model.plan:  # units whose mixers keep nothing still need a view
+            ctx.units.setdefault(e.cache, CacheUnitView())
+
+        logits = self.model.forward(ctx, view(4))
+        for e in entries:
+            cache.advance(e.handle, len(e.tokens))
+        return logits
+
+    def _upload(self, host: np.ndarray) -> torch.Tensor:
+        t = torch.from_numpy(host)
+        if self.env.device.type == "cpu":
+            return t
+        return t.pin_memory().to(self.env.device, non_blocking=True)

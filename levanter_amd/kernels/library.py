@@ -1,0 +1,236 @@
+"""Launchers of the HIP library: the only way the parts reach the GPU.
+
+Every method checks on the host that shapes, dtypes and strides are what the kernel and its
+grid assume, then calls the ``extern "C"`` entry point on the current stream. There is no CPU
+path: without a GPU or without the built library, ``get_kernels()`` raises.
+
+Conventions: the residual stream and logits are float32; norm weights, norm biases and linear
+biases are float32 vectors; matrices, tables, activations and the cache are in the compute
+dtype (bfloat16 or float32). A linear weight is ``[out, in]`` (each output's inputs contiguous).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+ACTIVATIONS = {"none": 0, "gelu_new": 1, "gelu": 2, "relu": 3, "silu": 4, "swish": 4, "quick_gelu": 5, "tanh": 6}
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+c_void_p, c_int, c_long, c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _req(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts) -> None:
+    for t in ts:
+        if t is not None:
+            _req(t.is_cuda, "a kernel was given a tensor that is not on the GPU")
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """Row stride (in elements) of a 2-D tensor whose rows are contiguous."""
+    _req(t.dim() == 2, f"{name} must have 2 dimensions, has {t.dim()}")
+    _req(t.shape[1] == 1 or t.stride(1) == 1, f"{name}: rows must be contiguous")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+class HipKernels:
+    """The built library, loaded."""
+
+    def __init__(self, path: str):
+        self.path = path
+        self.lib = ctypes.CDLL(path)
+        L = self.lib
+        L.lev_last_error.restype = ctypes.c_char_p
+        L.lev_abi_version.restype = c_int
+        sigs = {
+            "lev_embed": [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p],
+            "lev_norm": [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_int, c_void_p],
+            "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
+            "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+            "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
+            "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+            + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
+            "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 5 + [c_void_p],
+            "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                   c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 5 + [c_float, c_int, c_void_p],
+            "lev_attention_mfma_workspace": [c_int, c_int, c_int],
+        }
+        for name, args in sigs.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = c_long if name == "lev_attention_mfma_workspace" else c_int
+        self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
+
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.lev_last_error().decode())
+
+    # ---- embedding ---------------------------------------------------------------------
+    def embed(self, tokens, positions, table, pos_table, out) -> None:
+        """out[t] = table[tokens[t]] + pos_table[positions[t]] in float32. Ids are trusted (the step checks them)."""
+        _dev(tokens, positions, table, pos_table, out)
+        T, D = out.shape
+        _req(tokens.dtype == torch.int32 and positions.dtype == torch.int32, "embed: ids must be int32")
+        _req(tokens.numel() == T and positions.numel() == T, "embed: one token and one position per output row")
+        _req(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+        _req(table.is_contiguous() and table.shape[1] == D and table.dtype in _DT, "embed: bad table")
+        if pos_table is not None:
+            _req(pos_table.is_contiguous() and pos_table.shape[1] == D and pos_table.dtype == table.dtype, "embed: bad position table")
+        self._check(self.lib.lev_embed(_ptr(tokens), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(out), T, D,
+                                       _DT[table.dtype], _stream()))
+
+    # ---- norms ---------------------------------------------------------------------------
+    def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False) -> None:
+        """LayerNorm (or RMSNorm) of float32 rows into ``out`` (compute dtype). rows: int32 row indices into x."""
+        _dev(x, weight, bias, out, rows)
+        D = x.shape[1]
+        n = out.shape[0]
+        _req(x.dtype == torch.float32 and x.is_contiguous(), "norm: x must be contiguous float32")
+        _req(weight.dtype == torch.float32 and weight.numel() == D, "norm: weight must be float32 [D]")
+        _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == D), "norm: bias must be float32 [D]")
+        _req(out.is_contiguous() and out.shape[1] == D and out.dtype in _DT, "norm: bad out")
+        if rows is None:
+            _req(n == x.shape[0], "norm: out must have as many rows as x")
+        else:
+            _req(rows.dtype == torch.int32 and rows.numel() == n, "norm: rows must be int32, one per output row")
+        self._check(self.lib.lev_norm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(rows), n, D, float(eps), int(rms),
+                                      _DT[out.dtype], _stream()))
+
+    # ---- linear ----------------------------------------------------------------------------
+    def linear(self, a, w, bias, out, activation: str = "none", residual=None) -> None:
+        """out = act(a @ w.T + bias) (+ residual). a [M, K], w [N, K], out [M, N]; residual float32, may be ``out``."""
+        _dev(a, w, bias, out, residual)
+        M, K = a.shape
+        N = w.shape[0]
+        _req(w.dim() == 2 and w.shape[1] == K and w.is_contiguous(), f"linear: weight must be contiguous [N, {K}]")
+        _req(a.dtype == w.dtype and a.dtype in _DT, "linear: a and w must share a compute dtype")
+        _req(out.shape[0] == M and out.shape[1] == N and out.dtype in _DT, "linear: bad out")
+        _req(a.dtype == torch.bfloat16 or out.dtype == torch.float32, "linear: float32 inputs give float32 outputs")
+        _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()), "linear: bias must be float32 [N]")
+        lda, ldo = _rows(a, "linear: a"), _rows(out, "linear: out")
+        ldr = 0
+        if residual is not None:
+            _req(residual.dtype == torch.float32 and residual.shape == out.shape and out.dtype == torch.float32,
+                 "linear: a residual needs a float32 output of its shape")
+            ldr = _rows(residual, "linear: residual")
+        act = ACTIVATIONS[activation]
+        if a.dtype == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
+            self._check(self.lib.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
+                                                 M, N, K, act, _DT[out.dtype], _stream()))
+        else:
+            self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
+                                                   M, N, K, act, _DT[a.dtype], _DT[out.dtype], _stream()))
+
+    # ---- cache write -----------------------------------------------------------------------
+    def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int) -> None:
+        """Scatter the new tokens' keys and values ([T, n_kv_heads*head_dim] views) to ``dest[t] = page*page_size + offset``."""
+        _dev(k, v, k_pages, v_pages, dest)
+        T = k.shape[0]
+        _req(k.shape == v.shape and k.shape[1] == n_kv_heads * head_dim, "kv_write: k and v must be [T, kv_heads*head_dim]")
+        _req(k.dtype == v.dtype == k_pages.dtype == v_pages.dtype and k.dtype in _DT, "kv_write: dtypes differ")
+        _req(dest.dtype == torch.int32 and dest.numel() == T, "kv_write: one int32 destination per token")
+        _req(k_pages.is_contiguous() and v_pages.is_contiguous(), "kv_write: pages must be contiguous")
+        per_page = n_kv_heads * head_dim * page_size
+        _req(k_pages.numel() % per_page == 0 and k_pages.numel() == v_pages.numel(), "kv_write: page tensors do not fit the sizes")
+        self._check(self.lib.lev_kv_write(_ptr(k), _ptr(v), _rows(k, "kv_write: k"), _rows(v, "kv_write: v"), _ptr(k_pages),
+                                          _ptr(v_pages), _ptr(dest), T, n_kv_heads, head_dim, page_size, _DT[k.dtype], _stream()))
+
+    # ---- attention -------------------------------------------------------------------------
+    def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,
+                        page_size: int, scale: float, window: Optional[int], block_tables) -> None:
+        """Causal attention of the step's query tokens over the pages. ``meta`` is the step's
+        ``AttentionMeta`` (positions, token_seq and the work lists), block_tables int32 [S, B]."""
+        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq)
+        T = q.shape[0]
+        _req(q.shape[1] == n_heads * head_dim and out.shape == q.shape, "attention: q and out must be [T, heads*head_dim]")
+        _req(q.dtype == out.dtype == k_pages.dtype == v_pages.dtype and q.dtype in _DT, "attention: dtypes differ")
+        _req(meta.positions.numel() == T and meta.token_seq.numel() == T, "attention: one position and request row per token")
+        _req(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "attention: bad block tables")
+        _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
+        w = int(window) if window else 0
+        qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
+        if q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads):
+            splits = self.decode_splits(meta, n_heads, n_kv_heads)
+            need = self.lib.lev_attention_mfma_workspace(meta.n_decode * splits, n_heads, head_dim)
+            ws = meta.workspace(need, q.device)
+            self._check(self.lib.lev_attention_mfma(
+                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
+                _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles,
+                _ptr(meta.decode_tokens), meta.n_decode, _ptr(ws), n_heads, n_kv_heads, head_dim, page_size,
+                splits, float(scale), w, _stream()))
+        else:
+            self._check(self.lib.lev_attention_simple(
+                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
+                _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, page_size, float(scale), w,
+                _DT[q.dtype], _stream()))
+
+    @staticmethod
+    def decode_splits(meta, n_heads: int, n_kv_heads: int) -> int:
+        """Into how many key ranges a single-token query is split so that the chip is filled."""
+        if meta.n_decode == 0:
+            return 1
+        want = max(1, 2048 // max(1, meta.n_decode * n_kv_heads))
+        most = max(1, (meta.max_kv_len + 63) // 64)  # at least 64 keys per split
+        return int(min(want, most, 64))
+
+    @staticmethod
+    def mfma_attention_supports(head_dim: int, group: int) -> bool:
+        return head_dim % 16 == 0 and 16 <= head_dim <= 256 and group <= 16
+
+    # ---- sampling ----------------------------------------------------------------------------
+    def sample(self, logits, temperatures, keys, positions, out_tokens, out_logprobs) -> None:
+        """Greedy (temperature 0) or temperature sampling of float32 logits [R, V]; keys int32/uint32 [R, 2]."""
+        _dev(logits, temperatures, keys, positions, out_tokens, out_logprobs)
+        R, V = logits.shape
+        _req(logits.dtype == torch.float32, "sample: logits must be float32")
+        _req(temperatures.dtype == torch.float32 and temperatures.numel() == R, "sample: one float32 temperature per row")
+        _req(keys.dtype == torch.int32 and keys.numel() == 2 * R and keys.is_contiguous(), "sample: keys must be int32 [R, 2]")
+        _req(positions.dtype == torch.int32 and positions.numel() == R, "sample: one int32 position per row")
+        _req(out_tokens.dtype == torch.int32 and out_tokens.numel() == R, "sample: tokens out must be int32 [R]")
+        _req(out_logprobs.dtype == torch.float32 and out_logprobs.numel() == R, "sample: logprobs out must be float32 [R]")
+        self._check(self.lib.lev_sample(_ptr(logits), _rows(logits, "sample: logits"), _ptr(temperatures), _ptr(keys),
+                                        _ptr(positions), _ptr(out_tokens), _ptr(out_logprobs), R, V, _stream()))
+
+
+_KERNELS = None
+
+
+def set_kernels(k) -> None:
+    """Install a kernel library object (tests install a stand-in to run host logic without a GPU)."""
+    global _KERNELS
+    _KERNELS = k
+
+
+def get_kernels():
+    """The loaded HIP library. Raises when there is no GPU or the library cannot be built or loaded."""
+    global _KERNELS
+    if _KERNELS is None:
+        if not torch.cuda.is_available():
+            raise KernelError("levanter_amd runs on an AMD GPU only (torch.cuda.is_available() is False); there is no CPU path")
+        path = _build.ensure_built()
+        try:
+            _KERNELS = HipKernels(path)
+        except OSError as e:
+            raise KernelError(f"the HIP library {path} cannot be loaded: {e}") from None
+    return _KERNELS

@@ -1,0 +1,152 @@
+"""Interfaces of the parts and what a part sees of a step.
+
+Every part is built from ``(spec, tensors, env)``: its ``PartSpec`` (sizes and constants), a
+dict from its local parameter names to loaded tensors, and the ``BuildEnv`` (compute dtype,
+device, kernel library). No part knows which model it is in.
+
+The residual stream ``x`` is float32 ``[T, dim]`` in every precision; a norm turns it into the
+compute dtype ``h``; mixers and feed-forwards add their result to ``x`` in place.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from levanter_amd.parts.spec import PartSpec
+
+
+@dataclass
+class BuildEnv:
+    dtype: torch.dtype
+    device: torch.device
+    kernels: Any
+
+
+@dataclass
+class AttentionMeta:
+    """Device-side description of the step's tokens for the attention kernels."""
+
+    positions: torch.Tensor  # int32 [T] absolute position of each token
+    token_seq: torch.Tensor  # int32 [T] row of the step's block tables (= index of the request in the step)
+    prefill_tiles: Optional[torch.Tensor]  # int32 [n, 2]: first token and row count of each tile of a run longer than one token
+    n_prefill_tiles: int
+    decode_tokens: Optional[torch.Tensor]  # int32 [n]: tokens that are a run of their own
+    n_decode: int
+    max_kv_len: int  # the longest key range any token of the step reads
+    _workspaces: Dict[Any, torch.Tensor] = field(default_factory=dict)
+
+    def workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
+        if nbytes <= 0:
+            return None
+        ws = self._workspaces.get("ws")
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._workspaces["ws"] = ws
+        return ws
+
+
+@dataclass
+class GroupView:
+    """One cache group in this step."""
+
+    page_size: int
+    block_tables: torch.Tensor  # int32 [S, blocks]: page ids of the step's requests, -1 where none
+    dest: torch.Tensor  # int32 [T]: page * page_size + offset where each new token's keys and values go
+
+
+@dataclass
+class CacheUnitView:
+    """What a mixer gets of its cache unit in this step: pages (paged units) or state (slot units)."""
+
+    k_pages: Optional[torch.Tensor] = None
+    v_pages: Optional[torch.Tensor] = None
+    group: Optional[GroupView] = None
+    state: Optional[torch.Tensor] = None  # [slots, *shape]; rows ctx.seq_slots belong to the step's requests
+
+
+@dataclass
+class StepContext:
+    """What the parts see of one step. ``host`` holds the same facts as Python lists for parts that
+    steer from the host (run lengths, first positions, slots)."""
+
+    kernels: Any
+    dtype: torch.dtype
+    device: torch.device
+    n_tokens: int
+    tokens: torch.Tensor  # int32 [T]
+    attention: AttentionMeta
+    seq_slots: torch.Tensor  # int32 [S] state slot of each request in the step
+    host: Dict[str, Any]  # "run_lengths", "first_positions", "slots": lists, one entry per request in the step
+    units: Dict[int, CacheUnitView] = field(default_factory=dict)
+
+    def empty(self, rows: int, cols: int, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return torch.empty((rows, cols), dtype=dtype or self.dtype, device=self.device)
+
+
+class Part:
+    kind: str = ""
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        self.spec = spec
+        self.env = env
+
+
+class Norm(Part):
+    """``__call__(x_f32 [T, dim], ctx, rows=None) -> h [T or len(rows), dim]`` in the compute dtype."""
+
+    def __call__(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Two hooks; a position encoding uses one of them.
+
+    ``embedding_table()``: a table ``[positions, dim]`` whose row is added to the token embedding, or None.
+    ``rotate(q, k, ctx)``: change queries and keys in place before the cache write (identity by default).
+    ``max_positions``: the largest sequence length it allows, or None."""
+
+    max_positions: Optional[int] = None
+
+    def embedding_table(self) -> Optional[torch.Tensor]:
+        return None
+
+    def rotate(self, q: torch.Tensor, k: torch.Tensor, ctx: StepContext) -> None:
+        return None
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request.
+
+    ``cache_requirement()``: ``PagedKv``, ``SlotState`` or None: what one cache unit of it holds.
+    ``forward(h, x, ctx, unit, writes_cache)``: adds the mixer's output for ``h`` (compute dtype
+    ``[T, dim]``) to the residual ``x`` (float32 ``[T, dim]``) in place; reads (and, if
+    ``writes_cache``, first writes) ``unit``."""
+
+    def cache_requirement(self):
+        return None
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """``forward(h, x, ctx)``: adds the feed-forward's output for ``h`` to the residual ``x`` in place."""
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arranges two norms, a mixer and a feed-forward. ``forward(x, ctx, unit, writes_cache)`` updates ``x`` in place."""
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """``__call__(h [R, dim], ctx) -> logits float32 [R, vocab]``."""
+
+    def __call__(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError

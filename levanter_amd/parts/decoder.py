@@ -1,0 +1,128 @@
+"""DecoderLm: a runnable model built from a ``ModelSpec``.
+
+Embedding (token table + position encoding), layers of parts, the plan (the order in which
+layers run and which cache unit each reads), the final norm and the head. The reference wires
+the same sequence for paged decoding in src/levanter/models/llama.py:346-363,404-432,589-633
+(per-layer cache, logits from the packed positions); the GPT-2 mathematics is
+src/levanter/models/gpt2.py:237-248,268-273,345-362.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .base import BuildEnv, StepContext
+from .registry import BLOCKS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS
+from .spec import ModelSpec, PartSpec
+
+
+def _part_tensors(spec: PartSpec, tensors: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    out = {local: tensors[ts.name] for local, ts in spec.tensors.items()}
+    for v in spec.params.values():
+        if isinstance(v, PartSpec):  # a nested part's tensors travel under its own local names
+            out.update(_part_tensors(v, tensors))
+    return out
+
+
+class TokenEmbedding:
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        self.vocab_size = int(spec.params["vocab_size"])
+        self.dim = int(spec.params["dim"])
+        self.table = tensors[spec.tensors["table"].name].to(env.device, env.dtype).contiguous()
+        pos_spec: Optional[PartSpec] = spec.params.get("position")
+        self.position = None
+        if pos_spec is not None:
+            self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, _part_tensors(pos_spec, tensors), env)
+
+    @property
+    def max_positions(self) -> Optional[int]:
+        return None if self.position is None else self.position.max_positions
+
+    def __call__(self, ctx: StepContext) -> torch.Tensor:
+        x = ctx.empty(ctx.n_tokens, self.dim, torch.float32)
+        pos_table = None if self.position is None else self.position.embedding_table()
+        ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x)
+        return x
+
+
+class DecoderLm:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        self.spec = spec
+        self.env = env
+        self.vocab_size = spec.vocab_size
+        self.dim = spec.dim
+        self.embedding = TokenEmbedding(spec.embedding, tensors, env)
+        self.blocks = []
+        for layer in spec.layers:
+            norm1 = NORMS.get(layer.norm1.kind)(layer.norm1, _part_tensors(layer.norm1, tensors), env)
+            mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _part_tensors(layer.mixer, tensors), env)
+            norm2 = NORMS.get(layer.norm2.kind)(layer.norm2, _part_tensors(layer.norm2, tensors), env)
+            ff = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward, _part_tensors(layer.feed_forward, tensors), env)
+            self.blocks.append(BLOCKS.get(layer.block)(norm1, mixer, norm2, ff))
+        self.plan = list(spec.plan)
+        self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _part_tensors(spec.final_norm, tensors), env)
+        self.head = HEADS.get(spec.head.kind)(spec.head, _part_tensors(spec.head, tensors), env)
+        if hasattr(self.head, "tie"):
+            self.head.tie(self.embedding.table)
+        self._check_plan()
+
+    def _check_plan(self) -> None:
+        owners: Dict[int, int] = {}
+        for i, e in enumerate(self.plan):
+            if not 0 <= e.layer < len(self.blocks):
+                raise ValueError(f"plan entry {i} names layer {e.layer}, the model has {len(self.blocks)}")
+            if e.writes_cache:
+                if e.cache in owners:
+                    raise ValueError(f"plan entries {owners[e.cache]} and {i} both write cache unit {e.cache}")
+                owners[e.cache] = i
+        for i, e in enumerate(self.plan):
+            if not e.writes_cache:
+                if e.cache not in owners or owners[e.cache] > i:
+                    raise ValueError(f"plan entry {i} reads cache unit {e.cache} before any entry has written it")
+                a = self.blocks[self.plan[owners[e.cache]].layer].mixer.cache_requirement()
+                b = self.blocks[e.layer].mixer.cache_requirement()
+                if a != b:
+                    raise ValueError(f"plan entry {i} reads cache unit {e.cache}, whose owner keeps something else ({a} vs {b})")
+
+    @property
+    def max_positions(self) -> Optional[int]:
+        m = self.spec.max_positions
+        e = self.embedding.max_positions
+        if m is None:
+            return e
+        return m if e is None else min(m, e)
+
+    def cache_requirements(self) -> List[Tuple[int, object]]:
+        """(cache unit, requirement) of every unit that a plan entry writes."""
+        return [(e.cache, self.blocks[e.layer].mixer.cache_requirement()) for e in self.plan if e.writes_cache]
+
+    def forward(self, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
+        """Run the step's tokens through the plan; float32 logits ``[len(logit_rows), vocab]``."""
+        x = self.embedding(ctx)
+        for e in self.plan:
+            self.blocks[e.layer].forward(x, ctx, ctx.units[e.cache], e.writes_cache)
+        if logit_rows.numel() == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=ctx.device)
+        h = self.final_norm(x, ctx, rows=logit_rows)
+        return self.head(h, ctx)
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+        for obj in self._walk(self):
+            if isinstance(obj, torch.Tensor) and obj.data_ptr() not in seen:
+                seen.add(obj.data_ptr())
+                total += obj.numel() * obj.element_size()
+        return total
+
+    def _walk(self, obj, depth=0):
+        if isinstance(obj, torch.Tensor):
+            yield obj
+        elif isinstance(obj, (list, tuple)):
+            for o in obj:
+                yield from self._walk(o, depth + 1)
+        elif hasattr(obj, "__dict__") and depth < 6 and not isinstance(obj, (ModelSpec, PartSpec, BuildEnv)):
+            for k, v in vars(obj).items():
+                if k in ("spec", "env"):
+                    continue
+                yield from self._walk(v, depth + 1)

@@ -1,0 +1,28 @@
+"""A linear map as the parts hold it: the matrix ``[out, in]`` in the compute dtype, the bias in float32."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .base import BuildEnv, StepContext
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], layout: str, env: BuildEnv):
+        """``layout``: "in_out" (stored [in, out], as GPT-2 checkpoints do) or "out_in"."""
+        if layout not in ("in_out", "out_in"):
+            raise ValueError(f"unknown weight layout {layout!r}")
+        w = weight.to(env.device)
+        if layout == "in_out":
+            w = w.t()
+        self.weight = w.to(env.dtype).contiguous()  # [out, in]
+        self.bias = None if bias is None else bias.to(env.device, torch.float32).contiguous()
+        self.n_out, self.n_in = self.weight.shape
+
+    def __call__(self, a: torch.Tensor, ctx: StepContext, *, activation: str = "none", residual: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        if out is None:
+            out = residual if residual is not None else ctx.empty(a.shape[0], self.n_out, out_dtype)
+        ctx.kernels.linear(a, self.weight, self.bias, out, activation=activation, residual=residual)
+        return out
