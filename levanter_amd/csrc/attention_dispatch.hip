@@ -1,0 +1,44 @@
+// Entry point of the matrix-core attention: checks the sizes and calls the kernels of the head size.
+#include "common.h"
+
+#define LEV_DECL(HDV)                                                                                                       \
+  extern "C" int lev_attention_mfma_hd##HDV(const void*, long, void*, long, const void*, const void*, const int*, const int*, \
+                                            const int*, int, const int*, int, const int*, int, void*, int, int, int, int,    \
+                                            float, int, hipStream_t);
+LEV_DECL(16) LEV_DECL(32) LEV_DECL(48) LEV_DECL(64) LEV_DECL(80) LEV_DECL(96) LEV_DECL(112) LEV_DECL(128)
+#undef LEV_DECL
+
+// bytes of workspace for `rows` = decode tokens x splits partial results of H heads
+extern "C" long lev_attention_mfma_workspace(int rows, int H, int HD) {
+  return (long)rows * H * (HD + 2) * (long)sizeof(float);
+}
+
+extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
+
+extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long o_stride, const void* k_pages,
+                                  const void* v_pages, const int* positions, const int* token_seq, const int* block_tables,
+                                  int bt_stride, const int* prefill_tiles, int n_prefill_tiles, const int* decode_tokens,
+                                  int n_decode, void* workspace, int H, int KVH, int HD, int PS, int splits, float scale,
+                                  int window, hipStream_t stream) {
+  LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
+  LEV_REQUIRE(H / KVH <= 16, "attention (matrix cores): at most 16 query heads per kv head, got %d", H / KVH);
+  LEV_REQUIRE(HD % 16 == 0 && HD >= 16 && HD <= 128, "attention (matrix cores): head_dim=%d must be a multiple of 16 in 16..128", HD);
+  LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
+  LEV_REQUIRE(H <= 65535 && KVH <= 65535 && splits >= 1 && splits <= 65535, "attention: grid too large (heads=%d splits=%d)", H, splits);
+  LEV_REQUIRE(window >= 0, "attention: window=%d must not be negative", window);
+  LEV_REQUIRE(q_stride % 8 == 0 && o_stride % 4 == 0 && ((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
+              "attention (matrix cores): q rows must be 16-byte aligned and out rows 8-byte aligned");
+  LEV_REQUIRE(n_prefill_tiles == 0 || prefill_tiles, "attention: prefill tiles are missing");
+  LEV_REQUIRE(n_decode == 0 || decode_tokens, "attention: decode tokens are missing");
+  LEV_REQUIRE(n_decode == 0 || splits == 1 || workspace, "attention: split decoding needs a workspace");
+#define LEV_CASE(HDV)                                                                                                     \
+  case HDV:                                                                                                               \
+    return lev_attention_mfma_hd##HDV(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables,    \
+                                      bt_stride, prefill_tiles, n_prefill_tiles, decode_tokens, n_decode, workspace, H, KVH, \
+                                      PS, splits, scale, window, stream);
+  switch (HD) {
+    LEV_CASE(16) LEV_CASE(32) LEV_CASE(48) LEV_CASE(64) LEV_CASE(80) LEV_CASE(96) LEV_CASE(112) LEV_CASE(128)
+  }
+#undef LEV_CASE
+  return lev_fail("attention (matrix cores): no kernel for head_dim=%d", HD);
+}

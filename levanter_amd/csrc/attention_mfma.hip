@@ -1,0 +1,402 @@
+// Causal attention over the paged cache on the matrix cores, bfloat16 in, 32-bit softmax and
+// accumulation. Compiled once per head size: -DLEV_HD=<multiple of 16, at most 128>.
+//
+// Both kernels work on the transposed problem so that no operand needs a transposition:
+//   S^T = K . Q^T      A operand: 16 keys x 32 head dims (keys are rows), B operand: Q^T, in registers
+//   O^T = V^T . P^T    A operand: 16 head dims x 32 keys from the transposed value pages,
+//                      B operand: P^T, which is exactly what the lanes hold after the softmax
+// with the 16x16x32 MFMA: A lane l holds row l%16, k = 8*(l/16) .. +7; B lane l holds column l%16,
+// the same k; the accumulator's register r of lane l is row 4*(l/16) + r, column l%16.
+// The 16 rows of score tile (u, h) (u: which 32 keys of the block of 64, h: which half) are the keys
+// 32u + 8*(row/4) + 4h + row%4, so that lane group g = l/16 ends up with the probabilities of the
+// 8 consecutive keys 32u + 8g .. +7 in its two tiles: one k-slot run of the second product.
+//
+// Page layouts (elements): keys [page][kv_head][HD/8][PS][8], values [page][kv_head][HD][PS].
+//
+//   prefill kernel: one workgroup (4 waves) per (tile of up to 64 consecutive query tokens of one
+//                   request, head); keys and values of 64 positions at a time are staged in LDS.
+//   decode kernel:  one wave per (single-token query, kv head, split of the key range); operands go
+//                   from global memory straight into registers; the splits' partial results
+//                   (max, sum, unnormalised output) are merged in a fixed order by a second kernel.
+#include "common.h"
+
+#ifndef LEV_HD
+#error "compile with -DLEV_HD=<head size>"
+#endif
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define HD LEV_HD
+#define NCHUNK (HD / 8)            // 16-byte chunks of one key
+#define NKS ((HD + 31) / 32)       // k-steps of the score product
+#define NDT (HD / 16)              // 16-row tiles of O^T
+#define VS_STRIDE 72               // LDS row of V^T: 64 keys + 8 of padding (144 bytes)
+
+#define LEV_CAT_(a, b) a##b
+#define LEV_CAT(a, b) LEV_CAT_(a, b)
+#define LEV_NAME(base) LEV_CAT(base, LEV_HD)
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+}
+// key (0..63) of row i of score tile (u, h)
+__device__ __forceinline__ int tile_key(int u, int h, int i) { return 32 * u + 8 * (i >> 2) + 4 * h + (i & 3); }
+
+// One block of 64 keys for one wave: scores are in st[u][h] (S^T tiles, raw dot products).
+// Applies scale and mask, updates the running max m and sum l (per lane: column = query row),
+// rescales the output accumulators and returns the probabilities as B operands pf[u].
+// q_pos: position of this lane's query row (or -1 for a padding row); key0: position of key 0 of the block.
+__device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale, int q_pos, int lo, int key0, int g, float& m,
+                                              float& l, f32x4* o, u32x4 pf[2]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kp = key0 + 32 * u + 8 * g + 4 * h + r;
+        const bool ok = kp <= q_pos && kp >= lo;
+        const float s = ok ? st[u][h][r] * scale : -INFINITY;
+        st[u][h][r] = s;
+        mx = fmaxf(mx, s);
+      }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(m, mx);
+  const float base = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
+  const float corr = (m == -INFINITY) ? 0.f : __expf(m - base);
+  float psum = 0.f;
+  float p[2][2][4];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float e = __expf(st[u][h][r] - base);  // exp(-inf) = 0 for masked keys
+        p[u][h][r] = e;
+        psum += e;
+      }
+  l = l * corr + psum;
+  m = m_new;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) {
+    o[t][0] *= corr; o[t][1] *= corr; o[t][2] *= corr; o[t][3] *= corr;
+  }
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+    pf[u] = u32x4{pack_bf16(p[u][0][0], p[u][0][1]), pack_bf16(p[u][0][2], p[u][0][3]), pack_bf16(p[u][1][0], p[u][1][1]),
+                  pack_bf16(p[u][1][2], p[u][1][3])};
+}
+
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+                          const int* __restrict__ positions, const int* __restrict__ token_seq,
+                          const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int H, int KVH,
+                          int PS, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[4][NCHUNK][16][8];  // [score tile 2u+h][chunk][row][8]
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[HD][VS_STRIDE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 15, g = lane >> 4;
+  const int t0 = tiles[2 * blockIdx.x], rows = tiles[2 * blockIdx.x + 1];
+  const int h = blockIdx.y, kvh = h / (H / KVH);
+  const int pos0 = positions[t0];
+  const int* bt = block_tables + (size_t)token_seq[t0] * bt_stride;
+  const int my_row = wave * 16 + fr;
+  const int q_pos = my_row < rows ? pos0 + my_row : -1;
+  const int hi = pos0 + rows - 1;                                   // last key any row needs
+  const int lo_tile = window > 0 ? max(0, pos0 - window + 1) : 0;   // first key any row needs
+  const int lo = window > 0 ? max(0, q_pos - window + 1) : 0;       // first key this lane's row needs
+  const int wave_hi = min(hi, pos0 + wave * 16 + 15);
+  const bool wave_live = wave * 16 < rows;
+
+  // Q^T fragments of this lane's query row, kept for the whole kernel
+  u32x4 qf[NKS];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    const int c = 4 * s + g;
+    qf[s] = (q_pos >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(q + (size_t)(t0 + my_row) * q_stride + (size_t)h * HD + c * 8)
+                                        : u32x4{0, 0, 0, 0};
+  }
+  f32x4 o[NDT];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  constexpr int KCH = (64 * NCHUNK + 255) / 256;  // 16-byte chunks of K per thread and block
+  constexpr int VCH = (HD * 8 + 255) / 256;
+  u32x4 kr[KCH], vr[VCH];
+  const size_t head_elems = (size_t)HD * PS;
+  auto prefetch = [&](int kb) {
+    const int key0 = kb * 64;
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int x = tid + 256 * i;
+      const int kk = x & 63, c = x >> 6;
+      const int kp = key0 + kk;
+      u32x4 val = u32x4{0, 0, 0, 0};
+      if (c < NCHUNK && kp <= hi && kp >= lo_tile) {
+        const int page = bt[kp / PS];
+        if (page >= 0)
+          val = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)page * KVH + kvh) * head_elems + ((size_t)c * PS + kp % PS) * 8);
+      }
+      kr[i] = val;
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int y = tid + 256 * i;
+      const int j = y / (HD * 2), rem = y % (HD * 2);
+      const int d = rem >> 1, half = rem & 1;
+      const int kp = key0 + 16 * j + 8 * half;  // first of 8 keys; a page holds a multiple of 16
+      u32x4 val = u32x4{0, 0, 0, 0};
+      if (j < 4 && kp <= hi && kp + 7 >= lo_tile) {
+        const int page = bt[kp / PS];
+        if (page >= 0)
+          val = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)page * KVH + kvh) * head_elems + (size_t)d * PS + kp % PS);
+      }
+      vr[i] = val;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int x = tid + 256 * i;
+      const int kk = x & 63, c = x >> 6;
+      if (c < NCHUNK) {
+        const int tile = 2 * (kk >> 5) + ((kk & 7) >> 2);
+        const int row = 4 * ((kk & 31) >> 3) + (kk & 3);
+        *reinterpret_cast<u32x4*>(&Ks[tile][c][row][0]) = kr[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int y = tid + 256 * i;
+      const int j = y / (HD * 2), rem = y % (HD * 2);
+      if (j < 4) *reinterpret_cast<u32x4*>(&Vs[rem >> 1][16 * j + 8 * (rem & 1)]) = vr[i];
+    }
+  };
+
+  const int kb_first = lo_tile / 64, kb_last = hi / 64;
+  prefetch(kb_first);
+  for (int kb = kb_first; kb <= kb_last; ++kb) {
+    __syncthreads();  // everyone has finished reading the previous block
+    stage();
+    __syncthreads();
+    if (kb < kb_last) prefetch(kb + 1);
+    const int key0 = kb * 64;
+    if (!wave_live || key0 > wave_hi) continue;  // nothing in this block for this wave's rows
+    f32x4 st[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          const int c = 4 * s + g;
+          const u32x4 kf = c < NCHUNK ? *reinterpret_cast<const u32x4*>(&Ks[2 * u + hh][c][fr][0]) : u32x4{0, 0, 0, 0};
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
+        }
+        st[u][hh] = acc;
+      }
+    u32x4 pf[2];
+    softmax_block(st, scale, q_pos, lo, key0, g, m, l, o, pf);
+#pragma unroll
+    for (int t = 0; t < NDT; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vs[16 * t + fr][32 * u + 8 * g]);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[u]), o[t], 0, 0, 0);
+      }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (q_pos >= 0) {
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + (size_t)(t0 + my_row) * o_stride + (size_t)h * HD;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) {
+      const u32x2 v = u32x2{pack_bf16(o[t][0] * inv, o[t][1] * inv), pack_bf16(o[t][2] * inv, o[t][3] * inv)};
+      *reinterpret_cast<u32x2*>(orow + 16 * t + 4 * g) = v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode: one wave per (token, kv head, split). Columns of Q^T are the G = H / KVH query heads that
+// share the kv head. Partial results go to the workspace when there is more than one split:
+//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD]
+__global__ void __launch_bounds__(64)
+LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+                         const int* __restrict__ positions, const int* __restrict__ token_seq,
+                         const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ decode_tokens,
+                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o, int H, int KVH, int PS,
+                         int splits, float scale, int window) {
+  const int lane = threadIdx.x;
+  const int fr = lane & 15, g = lane >> 4;
+  const int idx = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+  const int t = decode_tokens[idx];
+  const int G = H / KVH;
+  const int pos = positions[t];
+  const int* bt = block_tables + (size_t)token_seq[t] * bt_stride;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kb_first = lo / 64, kb_last = pos / 64;
+  const int per = (kb_last - kb_first + 1 + splits - 1) / splits;
+  const int kb_begin = kb_first + z * per, kb_end = min(kb_last + 1, kb_begin + per);
+  const int head = kvh * G + fr;  // this lane's query head (column of Q^T)
+  const int q_pos = fr < G ? pos : -1;
+
+  u32x4 qf[NKS];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    const int c = 4 * s + g;
+    qf[s] = (q_pos >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(q + (size_t)t * q_stride + (size_t)head * HD + c * 8)
+                                        : u32x4{0, 0, 0, 0};
+  }
+  f32x4 o[NDT];
+#pragma unroll
+  for (int i = 0; i < NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const size_t head_elems = (size_t)HD * PS;
+
+  for (int kb = kb_begin; kb < kb_end; ++kb) {
+    const int key0 = kb * 64;
+    // key operands: tile (u, hh), row fr is key tile_key(u, hh, fr)
+    u32x4 kf[2][2][NKS];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kp = key0 + tile_key(u, hh, fr);
+        const bool ok = kp <= pos && kp >= lo;
+        const int page = ok ? bt[kp / PS] : -1;
+        const bf16_t* base = k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp % PS) * 8;
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          const int c = 4 * s + g;
+          kf[u][hh][s] = (page >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(base + (size_t)c * PS * 8) : u32x4{0, 0, 0, 0};
+        }
+      }
+    // value operands: tile dt, row fr is head dim 16*dt + fr, k-slots are keys 32u + 8g .. +7
+    u32x4 vf[NDT][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kp = key0 + 32 * u + 8 * g;
+      const bool ok = kp <= pos && kp + 7 >= lo;
+      const int page = ok ? bt[kp / PS] : -1;
+      const bf16_t* base = v_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + kp % PS;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        vf[dt][u] = page >= 0 ? *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS) : u32x4{0, 0, 0, 0};
+    }
+    f32x4 st[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NKS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][hh][s]), as_bf16x8(qf[s]), acc, 0, 0, 0);
+        st[u][hh] = acc;
+      }
+    u32x4 pf[2];
+    softmax_block(st, scale, q_pos, lo, key0, g, m, l, o, pf);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[dt][u]), as_bf16x8(pf[u]), o[dt], 0, 0, 0);
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (q_pos < 0) return;
+  if (splits == 1) {
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + (size_t)t * o_stride + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const u32x2 v = u32x2{pack_bf16(o[dt][0] * inv, o[dt][1] * inv), pack_bf16(o[dt][2] * inv, o[dt][3] * inv)};
+      *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * g) = v;
+    }
+  } else {
+    const size_t slot = ((size_t)idx * H + head) * splits + z;
+    if (g == 0) {
+      ws_m[slot] = m;
+      ws_l[slot] = l;
+    }
+    float* wo = ws_o + slot * HD;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(wo + 16 * dt + 4 * g) = o[dt];
+  }
+}
+
+// merge the splits of one (token, head) in the order of the splits
+__global__ void __launch_bounds__(64)
+LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __restrict__ decode_tokens,
+                          const float* __restrict__ ws_m, const float* __restrict__ ws_l, const float* __restrict__ ws_o,
+                          int H, int splits) {
+  const int idx = blockIdx.x, head = blockIdx.y;
+  const size_t slot0 = ((size_t)idx * H + head) * splits;
+  float mx = -INFINITY;
+  for (int z = 0; z < splits; ++z) mx = fmaxf(mx, ws_m[slot0 + z]);
+  float l = 0.f;
+  for (int z = 0; z < splits; ++z) {
+    const float mz = ws_m[slot0 + z];
+    if (mz != -INFINITY) l += ws_l[slot0 + z] * __expf(mz - mx);
+  }
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + (size_t)decode_tokens[idx] * o_stride + (size_t)head * HD;
+  for (int d = threadIdx.x; d < HD; d += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < splits; ++z) {
+      const float mz = ws_m[slot0 + z];
+      if (mz != -INFINITY) acc += ws_o[(slot0 + z) * HD + d] * __expf(mz - mx);
+    }
+    orow[d] = float_to_bf16(acc * inv);
+  }
+}
+
+extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, void* out, long o_stride, const void* k_pages,
+                                               const void* v_pages, const int* positions, const int* token_seq,
+                                               const int* block_tables, int bt_stride, const int* prefill_tiles,
+                                               int n_prefill_tiles, const int* decode_tokens, int n_decode, void* workspace,
+                                               int H, int KVH, int PS, int splits, float scale, int window,
+                                               hipStream_t stream) {
+  if (n_prefill_tiles > 0) {
+    dim3 grid(n_prefill_tiles, H);
+    LEV_NAME(attn_prefill_hd)<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
+                                                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq,
+                                                        block_tables, bt_stride, prefill_tiles, H, KVH, PS, scale, window);
+    if (int rc = lev_check_launch("attention prefill")) return rc;
+  }
+  if (n_decode > 0) {
+    const size_t rows = (size_t)n_decode * H * splits;
+    float* ws_m = (float*)workspace;
+    float* ws_l = ws_m + rows;
+    float* ws_o = ws_l + rows;
+    dim3 grid(n_decode, KVH, splits);
+    LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (const bf16_t*)k_pages,
+                                                      (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
+                                                      decode_tokens, ws_m, ws_l, ws_o, H, KVH, PS, splits, scale, window);
+    if (int rc = lev_check_launch("attention decode")) return rc;
+    if (splits > 1) {
+      dim3 cgrid(n_decode, H);
+      LEV_NAME(attn_combine_hd)<<<cgrid, 64, 0, stream>>>((bf16_t*)out, o_stride, decode_tokens, ws_m, ws_l, ws_o, H, splits);
+      if (int rc = lev_check_launch("attention combine")) return rc;
+    }
+  }
+  return 0;
+}

@@ -22,14 +22,17 @@ CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
 LIB_NAME = "liblevanter_amd_hip.so"
 ARCH = "gfx950"
 
+MFMA_ATTENTION_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
+
+# (source, extra defines, object name)
 SOURCES = [
-    "errors.hip",
-    "elementwise.hip",
-    "gemm_simple.hip",
-    "attention_simple.hip",
-    "gemm_mfma.hip",
-    "attention_mfma.hip",
-]
+    ("errors.hip", [], "errors.o"),
+    ("elementwise.hip", [], "elementwise.o"),
+    ("gemm_simple.hip", [], "gemm_simple.o"),
+    ("attention_simple.hip", [], "attention_simple.o"),
+    ("gemm_mfma.hip", [], "gemm_mfma.o"),
+    ("attention_dispatch.hip", [], "attention_dispatch.o"),
+] + [("attention_mfma.hip", [f"-DLEV_HD={hd}"], f"attention_mfma_hd{hd}.o") for hd in MFMA_ATTENTION_HEAD_DIMS]
 
 # -packed-fp32-ops off: packed 32-bit float instructions are not to be generated on this hardware pool
 HIPCC_FLAGS = [
@@ -117,16 +120,17 @@ def build(force: bool = True, jobs: Optional[int] = None) -> str:
     if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
         env["HOME"] = tempfile.gettempdir()  # hipcc wants a HOME it can write its caches to
     t0 = time.time()
-    _log(f"compiling {len(SOURCES)} HIP sources for {ARCH} with {jobs} jobs (first call only) ...")
+    _log(f"compiling {len(SOURCES)} HIP objects for {ARCH} with {jobs} jobs (first call only) ...")
 
-    def compile_one(src: str) -> str:
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    def compile_one(item) -> str:
+        src, defines, obj_name = item
+        obj = os.path.join(obj_dir, obj_name)
+        cmd = [hipcc, *HIPCC_FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
         t = time.time()
         r = subprocess.run(cmd, capture_output=True, text=True, env=env)
         if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}:\n{_filter(r.stderr)}")
-        _log(f"  {src} done in {time.time() - t:.0f}s")
+            raise RuntimeError(f"hipcc failed on {src} {' '.join(defines)}:\n{_filter(r.stderr)}")
+        _log(f"  {obj_name[:-2]} done in {time.time() - t:.0f}s")
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:

@@ -1,0 +1,275 @@
+"""Each HIP kernel alone against its plain statement in emulated_kernels.py, at sizes other than
+the engine's: odd vocabularies and widths, head sizes in steps of 16, groups of heads, windows."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from emulated_kernels import EmulatedKernels, gumbel_noise
+from helpers import dest_for, make_meta, random_block_tables
+
+pytestmark = pytest.mark.gpu
+
+EMU = EmulatedKernels()
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from levanter_amd.kernels import get_kernels
+
+    return get_kernels()
+
+
+def _rand(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def test_library_is_loaded(K):
+    assert K.path.endswith(".so")
+    assert K.lib.lev_abi_version() == 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D,V,P", [(1, 64, 50, 8), (7, 96, 1000, 33), (300, 1600, 257, 512)])
+def test_embed(K, dtype, T, D, V, P):
+    table, pos_table = _rand(V, D, dtype=dtype, seed=1), _rand(P, D, dtype=dtype, seed=2)
+    g = torch.Generator().manual_seed(3)
+    tok = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    pos = torch.randint(0, P, (T,), generator=g, dtype=torch.int32)
+    want = torch.empty(T, D)
+    EMU.embed(tok, pos, table, pos_table, want)
+    got = torch.empty(T, D, device=DEV)
+    K.embed(tok.to(DEV), pos.to(DEV), table.to(DEV), pos_table.to(DEV), got)
+    torch.testing.assert_close(got.cpu(), want, rtol=0, atol=0)
+    K.embed(tok.to(DEV), pos.to(DEV), table.to(DEV), None, got)
+    torch.testing.assert_close(got.cpu(), table[tok.long()].float(), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (33, 1600, 1e-5), (4, 4100, 1e-3)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_norm(K, out_dtype, T, D, eps, rms):
+    x = _rand(T, D, scale=3.0, seed=4) + 1.5
+    w, b = 1 + _rand(D, scale=0.1, seed=5), _rand(D, scale=0.1, seed=6)
+    want = torch.empty(T, D, dtype=out_dtype)
+    EMU.norm(x, w, b, eps, want, rms=rms)
+    got = torch.empty(T, D, dtype=out_dtype, device=DEV)
+    K.norm(x.to(DEV), w.to(DEV), b.to(DEV), eps, got, rms=rms)
+    tol = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    # gathered rows, no bias
+    rows = torch.tensor([T - 1, 0], dtype=torch.int32)
+    want2 = torch.empty(2, D, dtype=out_dtype)
+    EMU.norm(x, w, None, eps, want2, rows=rows, rms=rms)
+    got2 = torch.empty(2, D, dtype=out_dtype, device=DEV)
+    K.norm(x.to(DEV), w.to(DEV), None, eps, got2, rows=rows.to(DEV), rms=rms)
+    torch.testing.assert_close(got2.cpu().float(), want2.float(), **tol)
+
+
+def test_norm_constant_row_gives_bias(K):
+    x = torch.full((2, 96), 7.0)
+    w, b = _rand(96, seed=1), _rand(96, seed=2)
+    got = torch.empty(2, 96, device=DEV)
+    K.norm(x.to(DEV), w.to(DEV), b.to(DEV), 1e-5, got)
+    torch.testing.assert_close(got.cpu(), b.expand(2, 96), rtol=0, atol=1e-6)
+
+
+LINEAR_SHAPES = [(1, 64, 192), (2, 96, 320), (7, 320, 96), (16, 64, 1000), (17, 96, 50257 // 16), (64, 4096, 528),
+                 (65, 256, 257), (130, 96, 300), (300, 1600, 520), (257, 64, 50257 // 8)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,K_,N", LINEAR_SHAPES)
+def test_linear_plain_and_epilogues(K, dtype, M, K_, N):
+    a = _rand(M, K_, dtype=dtype, seed=1)
+    w = _rand(N, K_, dtype=dtype, scale=1 / math.sqrt(K_), seed=2)
+    bias = _rand(N, seed=3)
+    res = _rand(M, N, seed=4)
+    tol = dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    ad, wd, bd = a.to(DEV), w.to(DEV), bias.to(DEV)
+    # no epilogue, float32 out
+    want = torch.empty(M, N)
+    EMU.linear(a, w, None, want)
+    got = torch.empty(M, N, device=DEV)
+    K.linear(ad, wd, None, got)
+    torch.testing.assert_close(got.cpu(), want, rtol=2e-5 if dtype == torch.float32 else 1e-3, atol=2e-5 if dtype == torch.float32 else 1e-3)
+    # bias + activation, compute-dtype out
+    for act in ("gelu_new", "gelu"):
+        out_dtype = dtype
+        want = torch.empty(M, N, dtype=out_dtype)
+        EMU.linear(a, w, bias, want, activation=act)
+        got = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        K.linear(ad, wd, bd, got, activation=act)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    # bias + residual in place
+    want = torch.empty(M, N)
+    EMU.linear(a, w, bias, want, residual=res)
+    x = res.to(DEV).clone()
+    K.linear(ad, wd, bd, x, residual=x)
+    torch.testing.assert_close(x.cpu(), want, rtol=2e-5 if dtype == torch.float32 else 1e-3, atol=2e-5 if dtype == torch.float32 else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_strided_input_and_all_activations(K, dtype):
+    M, K_, N = 9, 96, 40
+    big = _rand(M, 3 * K_, dtype=dtype, seed=1)
+    a = big[:, K_:2 * K_]
+    w = _rand(N, K_, dtype=dtype, scale=0.1, seed=2)
+    for act in ("none", "relu", "silu", "quick_gelu", "tanh", "gelu", "gelu_new"):
+        want = torch.empty(M, N)
+        EMU.linear(a, w, None, want, activation=act)
+        got = torch.empty(M, N, device=DEV)
+        K.linear(big.to(DEV)[:, K_:2 * K_], w.to(DEV), None, got, activation=act)
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-3)
+
+
+def test_linear_bf16_picks_out_one_large_term(K):
+    # one large product among hundreds of small ones: a dropped or doubled k-step shows
+    M, K_, N = 3, 1024, 48
+    a = torch.full((M, K_), 1 / 64.0)
+    w = torch.full((N, K_), 1 / 64.0)
+    a[1, 777] = 8.0
+    w[5, 777] = 4.0
+    want = a @ w.t()
+    got = torch.empty(M, N, device=DEV)
+    K.linear(a.bfloat16().to(DEV), w.bfloat16().to(DEV), None, got)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-3, atol=1e-3)
+
+
+def test_linear_refuses_bad_sizes(K):
+    from levanter_amd.kernels import KernelError
+
+    a = torch.zeros(4, 100, dtype=torch.bfloat16, device=DEV)  # K not a multiple of 8: falls to the plain product
+    w = torch.zeros(8, 100, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(4, 8, device=DEV)
+    K.linear(a, w, None, out)
+    with pytest.raises(KernelError):
+        K.linear(a, torch.zeros(8, 96, dtype=torch.bfloat16, device=DEV), None, out)
+    with pytest.raises(KernelError):
+        K.linear(a.cpu(), w, None, out)
+
+
+def _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed):
+    """Random keys and values per request, written through the kv_write kernel into shuffled pages."""
+    bt = random_block_tables(kv_lens, PS, n_pages, seed, "cpu")
+    elems = KVH * HD * PS
+    kp = torch.zeros(n_pages, elems, dtype=dtype)
+    vp = torch.zeros(n_pages, elems, dtype=dtype)
+    kd, vd = kp.to(DEV), vp.to(DEV)
+    ks, vs = [], []
+    for s, n in enumerate(kv_lens):
+        k = _rand(n, KVH * HD, dtype=dtype, seed=seed * 100 + s)
+        v = _rand(n, KVH * HD, dtype=dtype, seed=seed * 100 + 50 + s)
+        dest = torch.tensor(dest_for(bt, s, range(n), PS), dtype=torch.int32)
+        EMU.kv_write(k, v, kp, vp, dest, KVH, HD, PS)
+        K.kv_write(k.to(DEV), v.to(DEV), kd, vd, dest.to(DEV), KVH, HD, PS)
+        ks.append(k)
+        vs.append(v)
+    torch.testing.assert_close(kd.cpu(), kp, rtol=0, atol=0)
+    torch.testing.assert_close(vd.cpu(), vp, rtol=0, atol=0)
+    return bt, kp, vp, kd, vd, ks, vs
+
+
+ATTN_CASES = [
+    # (H, KVH, HD, PS, runs=(q_len, kv_len), window)
+    (4, 4, 16, 16, [(8, 8)], None),
+    (3, 3, 32, 16, [(8, 8), (32, 32), (16, 16)], None),
+    (2, 1, 64, 16, [(1, 10), (3, 37), (9, 64)], None),
+    (4, 2, 96, 32, [(34, 34), (17, 17)], None),
+    (5, 5, 128, 16, [(1, 9), (1, 10), (1, 34), (1, 17)], None),
+    (2, 2, 48, 16, [(64, 64), (1, 10), (37, 37)], None),
+    (8, 2, 80, 64, [(5, 5), (15, 15), (25, 25), (35, 35), (45, 45)], None),
+    (4, 4, 112, 16, [(5, 47), (2, 130), (1, 200), (70, 150)], None),
+    (4, 1, 128, 16, [(1, 300), (130, 260)], 50),
+    (3, 3, 32, 16, [(1, 100), (20, 90), (1, 7)], 16),
+    (2, 2, 256, 16, [(1, 40), (9, 33)], None),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KVH,HD,PS,runs,window", ATTN_CASES)
+def test_paged_attention(K, dtype, H, KVH, HD, PS, runs, window):
+    kv_lens = [k for _, k in runs]
+    n_pages = sum((k + PS - 1) // PS for k in kv_lens) + 3
+    bt, kp, vp, kd, vd, ks, vs = _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed=7)
+    T = sum(q for q, _ in runs)
+    q = _rand(T, H * HD, dtype=dtype, seed=11)
+    scale = 1 / math.sqrt(HD) / 2
+    meta_c = make_meta(runs, "cpu")
+    want = torch.empty(T, H * HD, dtype=dtype)
+    EMU.paged_attention(q, want, kp, vp, meta_c, n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=scale,
+                        window=window, block_tables=bt)
+    meta = make_meta(runs, DEV)
+    got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q.to(DEV), got, kd, vd, meta, n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=scale,
+                      window=window, block_tables=bt.to(DEV))
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key(K, dtype):
+    # among 700 keys one (far back, in the middle of a page) matches the query strongly: the output is its value
+    H = KVH = 2
+    HD, PS, n = 64, 16, 700
+    bt = random_block_tables([n], PS, 60, 3, "cpu")
+    k = _rand(n, KVH * HD, dtype=torch.float32, scale=0.05, seed=1)
+    v = _rand(n, KVH * HD, dtype=torch.float32, seed=2)
+    q = _rand(1, H * HD, dtype=torch.float32, scale=0.05, seed=3)
+    target = 217
+    k[target, :HD] = 3.0
+    q[0, :HD] = 3.0  # head 0 only: score 64 * 9 * scale
+    kd = torch.zeros(60, KVH * HD * PS, dtype=dtype, device=DEV)
+    vd = torch.zeros_like(kd)
+    dest = torch.tensor(dest_for(bt, 0, range(n), PS), dtype=torch.int32, device=DEV)
+    K.kv_write(k.to(dtype).to(DEV), v.to(dtype).to(DEV), kd, vd, dest, KVH, HD, PS)
+    for runs in ([(1, n)], [(5, n)]):
+        T = runs[0][0]
+        qq = q.expand(T, -1).contiguous()
+        got = torch.empty(T, H * HD, dtype=dtype, device=DEV)
+        K.paged_attention(qq.to(dtype).to(DEV), got, kd, vd, make_meta(runs, DEV), n_heads=H, n_kv_heads=KVH, head_dim=HD,
+                          page_size=PS, scale=1 / 8.0, window=None, block_tables=bt.to(DEV))
+        torch.testing.assert_close(got[:, :HD].cpu().float(), v[target, :HD].to(dtype).float().expand(T, -1), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("temp", [0.0, 0.7, 1.3])
+@pytest.mark.parametrize("R,V", [(1, 5), (3, 1000), (4, 50257)])
+def test_sample(K, temp, R, V):
+    logits = _rand(R, V, scale=2.0, seed=5)
+    temps = torch.full((R,), temp)
+    keys = torch.tensor([[r * 7 + 1, r * 13 + 5] for r in range(R)], dtype=torch.int32)
+    pos = torch.tensor([r * 3 + 2 for r in range(R)], dtype=torch.int32)
+    want_t, want_l = torch.empty(R, dtype=torch.int32), torch.empty(R)
+    EMU.sample(logits, temps, keys, pos, want_t, want_l)
+    got_t = torch.empty(R, dtype=torch.int32, device=DEV)
+    got_l = torch.empty(R, device=DEV)
+    K.sample(logits.to(DEV), temps.to(DEV), keys.to(DEV), pos.to(DEV), got_t, got_l)
+    assert got_t.cpu().tolist() == want_t.tolist()
+    torch.testing.assert_close(got_l.cpu(), want_l, rtol=1e-4, atol=1e-4)
+
+
+def test_sample_ties_and_frequencies(K):
+    logits = torch.zeros(2, 9)
+    logits[0, [2, 6]] = 1.0  # a tie: the lowest index wins
+    got_t = torch.empty(2, dtype=torch.int32, device=DEV)
+    got_l = torch.empty(2, device=DEV)
+    z = torch.zeros(2, dtype=torch.int32, device=DEV)
+    K.sample(logits.to(DEV), torch.zeros(2, device=DEV), torch.zeros(2, 2, dtype=torch.int32, device=DEV), z, got_t, got_l)
+    assert got_t.cpu().tolist() == [2, 0]
+    # frequencies over many keys follow softmax(logits / T)
+    base = torch.tensor([0.1, 2.0, -1.0, 1.9, 0.0])
+    n, t = 20000, 0.7
+    lg = base.expand(n, 5).contiguous().to(DEV)
+    keys = torch.stack([torch.arange(n, dtype=torch.int32), torch.full((n,), 12345, dtype=torch.int32)], 1).to(DEV)
+    toks = torch.empty(n, dtype=torch.int32, device=DEV)
+    lps = torch.empty(n, device=DEV)
+    K.sample(lg, torch.full((n,), t, device=DEV), keys, torch.zeros(n, dtype=torch.int32, device=DEV), toks, lps)
+    freq = torch.bincount(toks.cpu().long(), minlength=5).float() / n
+    p = torch.softmax(base / t, -1)
+    assert bool(((freq - p).abs() < 4 * torch.sqrt(p * (1 - p) / n)).all()), (freq, p)
+    # the noise is the documented function of (key, position, entry)
+    noise = gumbel_noise(3, 12345, 0, 5)
+    assert int(toks[3]) == int(torch.argmax(base / t + noise))
