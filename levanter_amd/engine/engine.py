@@ -1,0 +1,146 @@
+"""InferenceEngine: the Python entry point. From requests to generated tokens.
+
+Reference: ``InferenceEngine.from_model_with_config`` / ``.generate(requests) -> GenerationResult``
+/ ``.reset()`` (src/levanter/inference/engine.py:705-776,1019-1199). Returned tokens are the
+generated ones only, the stopping token included (engine.py:613,
+tests/inference/test_engine.py:87-92), ordered by request and generation (engine.py:1173-1190).
+"""
+from __future__ import annotations
+
+import logging
+import time
+from typing import List, Optional, Sequence
+
+import torch
+
+from levanter_amd.config import InferenceEngineConfig, LmConfig
+from levanter_amd.parts import BuildEnv, DecoderLm
+from levanter_amd.sampling import Sampler, fold_in, make_key
+
+from .loading import load_model, make_cache, make_env, random_model
+from .request import GenerationResult, Request, SeqDecodingParams
+from .scheduler import PlannedEntry, Scheduler, Sequence_
+from .step import ModelRunner, StepEntry
+
+logger = logging.getLogger(__name__)
+
+__all__ = ["InferenceEngine", "Request", "SeqDecodingParams", "GenerationResult", "InferenceEngineConfig"]
+
+
+class InferenceEngine:
+    def __init__(self, model, config: InferenceEngineConfig, env: BuildEnv, allocate: bool = True):
+        self.model = model
+        self.config = config
+        self.env = env
+        self.cache = make_cache(model, config)
+        self.runner = ModelRunner(model, self.cache, env, allocate=allocate)
+        self.sampler = Sampler(env.kernels, env.device)
+        self.scheduler = Scheduler(self.cache, config, self.runner.max_len)
+        self.stats = {"steps": 0, "tokens_in": 0, "device_s": 0.0}
+
+    # ---- construction -------------------------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, model_dir: str, config: Optional[InferenceEngineConfig] = None, device: Optional[str] = None):
+        """Load ``config.json`` and ``model.safetensors`` of a folder; the architecture comes from the registry."""
+        config = config or InferenceEngineConfig()
+        env = make_env(config.compute_dtype, device)
+        _, model = load_model(model_dir, env)
+        return cls(model, config, env)
+
+    @classmethod
+    def from_config(cls, model_config: LmConfig, seed: int = 0, config: Optional[InferenceEngineConfig] = None,
+                    device: Optional[str] = None):
+        """A model with random weights drawn on the GPU from ``seed``."""
+        config = config or InferenceEngineConfig()
+        env = make_env(config.compute_dtype, device)
+        return cls(random_model(model_config, seed, env), config, env)
+
+    @classmethod
+    def from_model_with_config(cls, model: DecoderLm, tokenizer=None, config: Optional[InferenceEngineConfig] = None):
+        """The reference's constructor name (engine.py:705-731); the tokenizer is not needed: token ids in and out."""
+        return cls(model, config or InferenceEngineConfig(), model.env)
+
+    # ---- requests ---------------------------------------------------------------------------------
+    def _validate(self, requests: Sequence[Request]) -> None:
+        cfg = self.config
+        v = self.model.vocab_size
+        for r in requests:
+            if r.n_generations < 1 or r.n_generations > cfg.max_seqs:
+                raise ValueError(f"request {r.request_id}: n_generations={r.n_generations} must be in 1..max_seqs={cfg.max_seqs}")
+            if len(r.prompt_tokens) == 0:
+                raise ValueError(f"request {r.request_id}: empty prompt")
+            if len(r.prompt_tokens) >= self.runner.max_len:
+                raise ValueError(f"request {r.request_id}: a prompt of {len(r.prompt_tokens)} tokens leaves no room under the "
+                                 f"limit of {self.runner.max_len} (model positions and page_size * max_pages_per_seq)")
+            bad = [t for t in r.prompt_tokens if not 0 <= t < v]
+            if bad:
+                raise ValueError(f"request {r.request_id}: token id {bad[0]} is outside the vocabulary of {v}")
+            stops = r.decode_params.stop_tokens
+            if stops is not None:
+                if len(stops) > cfg.max_stop_seqs:
+                    raise ValueError(f"request {r.request_id}: {len(stops)} stop sequences, max_stop_seqs={cfg.max_stop_seqs}")
+                if any(len(s) > cfg.max_stop_tokens for s in stops):
+                    raise ValueError(f"request {r.request_id}: a stop sequence is longer than max_stop_tokens={cfg.max_stop_tokens}")
+            if r.enable_logprobs and not cfg.enable_logprobs:
+                raise ValueError(f"request {r.request_id} asks for logprobs but the engine has enable_logprobs=False")
+
+    def enqueue_requests(self, requests: Sequence[Request]) -> List[Sequence_]:
+        self._validate(requests)
+        seqs = []
+        for r in requests:
+            k = r.decode_params.key
+            base = fold_in(make_key(self.config.seed), r.request_id) if k is None else (make_key(k) if isinstance(k, int) else tuple(k))
+            for child in range(r.n_generations):
+                key = base if r.n_generations == 1 else fold_in(base, child)
+                seq = Sequence_(request=r, child=child, key=key, order=self.scheduler.next_order(),
+                                tokens=list(r.prompt_tokens), prompt_len=len(r.prompt_tokens))
+                self.scheduler.add(seq)
+                seqs.append(seq)
+        return seqs
+
+    # ---- one scheduler iteration -----------------------------------------------------------------------
+    def step(self) -> List[Sequence_]:
+        """Plan a step, run it, sample, commit. Returns the sequences that finished in it."""
+        plan: List[PlannedEntry] = self.scheduler.plan()
+        if not plan:
+            return []
+        entries = [StepEntry(e.seq.handle, e.tokens, [len(e.tokens) - 1] if e.wants_logits else []) for e in plan]
+        t0 = time.perf_counter()
+        logits = self.runner.step(entries)
+        wanted = [e for e in plan if e.wants_logits]
+        toks: List[int] = []
+        lps: List[float] = []
+        if wanted:
+            temps = [e.seq.request.decode_params.temperature for e in wanted]
+            keys = [e.seq.key for e in wanted]
+            positions = [e.seq.n_cached - 1 for e in wanted]  # position of the token whose logits are sampled
+            t, lp = self.sampler(logits, temps, keys, positions)
+            toks = t.cpu().tolist()
+            lps = lp.cpu().tolist()
+        self.stats["steps"] += 1
+        self.stats["tokens_in"] += sum(len(e.tokens) for e in plan)
+        self.stats["device_s"] += time.perf_counter() - t0
+        return self.scheduler.commit(plan, toks, lps)
+
+    def generate(self, requests: Sequence[Request]) -> GenerationResult:
+        seqs = self.enqueue_requests(requests)
+        t0 = time.perf_counter()
+        idle_steps = 0
+        while not all(s.done for s in seqs):
+            n_before = self.stats["steps"]
+            self.step()
+            idle_steps = idle_steps + 1 if self.stats["steps"] == n_before else 0
+            if idle_steps >= 2:  # the reference breaks after two iterations without progress (engine.py:1160-1171)
+                raise RuntimeError("the scheduler made no step twice in a row although requests are unfinished")
+        dt = time.perf_counter() - t0
+        total = sum(len(s.generated) for s in seqs)
+        logger.info("generated %d tokens in %.3fs (%.1f tok/s)", total, dt, total / max(dt, 1e-9))
+        want_lp = self.config.enable_logprobs and any(s.request.enable_logprobs for s in seqs)
+        return GenerationResult(tokens=[list(s.generated) for s in seqs],
+                                logprobs=[list(s.logprobs) for s in seqs] if want_lp else None,
+                                total_generated=total, finish_reasons=[s.finish_reason for s in seqs])
+
+    def reset(self) -> None:
+        """Drop every request and give back all pages and slots (engine.py:761-776)."""
+        self.scheduler.abort_all()
+        self.cache.reset()

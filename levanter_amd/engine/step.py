@@ -168,7 +168,8 @@ class ModelRunner:
                        for gi in range(n_groups)]
         for unit, g in cache.group_of_unit.items():
             i = g.unit_pos[unit]
-            ctx.units[unit] = CacheUnitView(k_pages=g.k_pages[i], v_pages=g.v_pages[i], group=group_views[g.index])
+            ctx.units[unit] = CacheUnitView(k_pages=None if g.k_pages is None else g.k_pages[i],
+                                            v_pages=None if g.v_pages is None else g.v_pages[i], group=group_views[g.index])
         for unit, t in cache.state.tensors.items():
             ctx.units[unit] = CacheUnitView(state=t)
         for e in self.model.plan:  # units whose mixers keep nothing still need a view

@@ -196,7 +196,7 @@ class HipKernels:
 
     @staticmethod
     def mfma_attention_supports(head_dim: int, group: int) -> bool:
-        return head_dim % 16 == 0 and 16 <= head_dim <= 256 and group <= 16
+        return head_dim % 16 == 0 and 16 <= head_dim <= 128 and group <= 16
 
     # ---- sampling ----------------------------------------------------------------------------
     def sample(self, logits, temperatures, keys, positions, out_tokens, out_logprobs) -> None:

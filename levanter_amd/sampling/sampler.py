@@ -1,0 +1,65 @@
+"""Greedy and temperature sampling on the GPU.
+
+Reference: ``Sampler`` (src/levanter/layers/sampler.py:15-81): logits in 32-bit; temperature 0
+gives the argmax, otherwise a categorical draw from ``logits / temperature``; the log-probability
+of the chosen token is ``scaled_logit - logsumexp(scaled_logits)``. The reference samples with
+``fold_in(request key, position of the input token)`` (src/levanter/inference/jit_scheduler.py:141-156),
+so a token's randomness depends on the request and the position only, not on the batch. Here the
+draw is argmax(scaled logits + Gumbel noise) with noise from a counter-based generator keyed by
+(request key, position, vocabulary entry). The reference has no top-k, top-p or penalties.
+"""
+from __future__ import annotations
+
+from typing import Sequence, Tuple
+
+import numpy as np
+import torch
+
+_MASK64 = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK64
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK64
+    return z ^ (z >> 31)
+
+
+def make_key(seed: int) -> Tuple[int, int]:
+    """A 64-bit sampling key (two 32-bit words) from an integer seed (the reference's ``PRNGKey(seed)``)."""
+    z = _splitmix64(int(seed) & _MASK64)
+    return z & 0xFFFFFFFF, z >> 32
+
+
+def fold_in(key: Tuple[int, int], data: int) -> Tuple[int, int]:
+    """A new key from a key and an integer (the reference's ``jax.random.fold_in``; not the same bits)."""
+    z = _splitmix64(((key[1] << 32) | key[0]) ^ _splitmix64(int(data) & _MASK64))
+    return z & 0xFFFFFFFF, z >> 32
+
+
+def _as_i32(word: int) -> int:
+    return word - (1 << 32) if word >= (1 << 31) else word
+
+
+class Sampler:
+    def __init__(self, kernels, device):
+        self.kernels = kernels
+        self.device = torch.device(device)
+
+    def __call__(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[Tuple[int, int]],
+                 positions: Sequence[int]) -> Tuple[torch.Tensor, torch.Tensor]:
+        """logits float32 [R, V] on the device; one temperature, key and position per row.
+        Returns (tokens int32 [R], log-probabilities float32 [R]) on the device."""
+        r = logits.shape[0]
+        assert len(temperatures) == len(keys) == len(positions) == r
+        host = np.empty(4 * r, np.int32)
+        host[:r] = np.asarray(temperatures, np.float32).view(np.int32)
+        host[r:3 * r] = np.asarray([[_as_i32(k[0]), _as_i32(k[1])] for k in keys], np.int64).reshape(-1)
+        host[3 * r:] = np.asarray(positions, np.int64)
+        t = torch.from_numpy(host)
+        dev = t if self.device.type == "cpu" else t.pin_memory().to(self.device, non_blocking=True)
+        tokens = torch.empty(r, dtype=torch.int32, device=self.device)
+        logprobs = torch.empty(r, dtype=torch.float32, device=self.device)
+        self.kernels.sample(logits, dev[:r].view(torch.float32), dev[r:3 * r].view(r, 2), dev[3 * r:], tokens, logprobs)
+        return tokens, logprobs

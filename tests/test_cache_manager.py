@@ -1,0 +1,153 @@
+"""The cache manager on the host: no page lost, held twice or freed twice, under random orders of
+requests; groups with and without a window; slots of fixed-size state."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from levanter_amd.cache import NO_PAGE, CacheManager, OutOfPages, OutOfSlots, PagedKv, PagePool, SlotState
+
+
+def make(n_pages=8, page_size=16, max_seqs=4, max_pages_per_seq=8, window=None, extra=()):
+    reqs = [(0, PagedKv(2, 16)), (1, PagedKv(2, 16))]
+    if window:
+        reqs.append((2, PagedKv(2, 16, window=window)))
+    reqs += list(extra)
+    return CacheManager(reqs, n_pages=n_pages, page_size=page_size, max_seqs=max_seqs, max_pages_per_seq=max_pages_per_seq)
+
+
+def test_pool_refuses_double_free_and_counts():
+    p = PagePool(3)
+    a, b = p.alloc(), p.alloc()
+    assert (a, b) == (0, 1) and p.n_free == 1
+    p.free(a)
+    with pytest.raises(RuntimeError, match="freed twice"):
+        p.free(a)
+    assert p.alloc() == a  # the page freed last is handed out first
+    p.alloc()
+    with pytest.raises(OutOfPages):
+        p.alloc()
+    p.check()
+
+
+def test_units_with_equal_needs_share_a_group():
+    c = make(window=40)
+    assert len(c.groups) == 2
+    assert c.groups[0].units == [0, 1] and c.groups[1].units == [2] and c.groups[1].requirement.window == 40
+    assert c.group_of_unit[1] is c.groups[0]
+
+
+def test_pages_come_lazily_and_go_back_on_close():
+    # as the reference's page table (page_table.py:142-275): a page is taken when a token first lands on it
+    c = make()
+    h = c.open("a")
+    assert h.slot == 0 and c.pages_needed(h, 16) == 1 and c.pages_needed(h, 17) == 2
+    c.extend(h, 5)
+    c.advance(h, 5)
+    assert c.groups[0].pages_held(h.slot) == [0] and h.length == 5
+    c.extend(h, 11)
+    c.advance(h, 11)  # 16 tokens: still one page
+    assert c.groups[0].pages_held(h.slot) == [0]
+    c.extend(h, 1)
+    c.advance(h, 1)
+    assert c.groups[0].pages_held(h.slot) == [0, 1]
+    assert c.destination(c.groups[0], h, 16) == 1 * 16 + 0 and c.destination(c.groups[0], h, 7) == 7
+    c.check_invariants()
+    c.close(h)
+    assert c.groups[0].pool.n_free == 8 and (c.groups[0].block_tables == NO_PAGE).all()
+    with pytest.raises(RuntimeError, match="closed twice"):
+        c.close(h)
+    c.check_invariants()
+
+
+def test_extend_is_all_or_nothing():
+    c = make(n_pages=3, window=1000)
+    a, b = c.open("a"), c.open("b")
+    c.extend(a, 32)
+    c.advance(a, 32)
+    before = [g.pool.n_free for g in c.groups]
+    assert not c.can_extend(b, 40)
+    with pytest.raises(OutOfPages):
+        c.extend(b, 40)
+    assert [g.pool.n_free for g in c.groups] == before
+    assert all(g.pages_held(b.slot) == [] for g in c.groups)
+    c.check_invariants()
+    with pytest.raises(ValueError, match="max_pages_per_seq"):
+        c.extend(a, 16 * 8)
+
+
+def test_slots_run_out_and_come_back():
+    c = make(max_seqs=2)
+    a, b = c.open("a"), c.open("b")
+    with pytest.raises(OutOfSlots):
+        c.open("c")
+    c.close(a)
+    assert c.open("c").slot == a.slot
+
+
+def test_window_group_gives_pages_back_while_the_request_runs():
+    c = make(n_pages=6, window=20, max_pages_per_seq=32)
+    g_all, g_win = c.groups
+    h = c.open("a")
+    held = []
+    for _ in range(80):  # one token at a time up to 80 tokens
+        c.extend(h, 1)
+        c.advance(h, 1)
+        c.check_invariants()
+        held.append(len(g_win.pages_held(h.slot)))
+    assert len(g_all.pages_held(h.slot)) == 5
+    assert max(held) <= 3  # 20 keys span at most 3 pages of 16
+    # the next query (position 80) reads keys 61..80: blocks 0..2 are gone, block 3 (48..63) is still there
+    assert (g_win.block_tables[h.slot, :3] == NO_PAGE).all() and g_win.block_tables[h.slot, 3] != NO_PAGE
+    c.close(h)
+    c.check_invariants()
+    assert g_win.pool.n_free == 6
+
+
+def test_state_slots_are_zeroed_on_admission():
+    c = make(extra=[(5, SlotState((3, 2)))])
+    c.allocate_tensors(torch.float32, "cpu")
+    assert c.state.tensors[5].shape == (4, 3, 2)
+    a = c.open("a")
+    c.state.tensors[5][a.slot] += 7
+    c.close(a)
+    b = c.open("b")
+    assert b.slot == a.slot and float(c.state.tensors[5][b.slot].abs().sum()) == 0.0
+    k, v, g = c.unit_pages(1)
+    assert k.shape == (8, 2 * 16 * 16) and g is c.groups[0]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_of_requests_keep_the_books(seed):
+    rng = random.Random(seed)
+    c = make(n_pages=12, max_seqs=4, max_pages_per_seq=6, window=24 if seed % 2 else None)
+    live = {}
+    n_out_of_pages = 0
+    for step in range(400):
+        op = rng.random()
+        if op < 0.25 and c.n_free_slots:
+            h = c.open(step)
+            live[step] = h
+        elif op < 0.85 and live:
+            h = live[rng.choice(list(live))]
+            n = rng.choice([1, 1, 1, 2, 7, 16, 33])
+            if h.length + n > 16 * 6:
+                continue
+            try:
+                c.extend(h, n)
+                c.advance(h, n)
+            except OutOfPages:
+                n_out_of_pages += 1
+        elif live:
+            c.close(live.pop(rng.choice(list(live))))
+        c.check_invariants()
+        for g in c.groups:
+            held = sum(len(g.pages_held(s)) for s in range(c.max_seqs))
+            assert held + g.pool.n_free == g.pool.n_pages  # no page lost
+            pages = [p for s in range(c.max_seqs) for p in g.pages_held(s)]
+            assert len(pages) == len(set(pages))  # none held twice
+    assert n_out_of_pages > 0  # the pool was small enough to run out
+    c.reset()
+    c.check_invariants()
+    assert all(g.pool.n_free == g.pool.n_pages for g in c.groups) and c.n_free_slots == 4

@@ -1,0 +1,80 @@
+"""Replay through bin/trace_run on the GPU, in 32-bit and in bfloat16: the same requests whole,
+with the last 32 tokens one by one, in portions of changing size, and mixed with other requests in
+a pool so small that pages are used again. All compared with the plain implementation."""
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2 as P
+import traces as TR
+from helpers import read_weights, write_model
+from tiny_configs import TINY
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# 32-bit: differences of summation order only (the reference's own tolerance for paged attention on
+# the CPU is 1e-4, tests/inference/test_paged_attention.py:140-142).
+TOL_F32 = dict(rtol=1e-4, atol=1e-5)
+# bfloat16 against the plain implementation that rounds to bfloat16 at the same places: what is left
+# are accumulation order and roundings that fall on the other side (one bfloat16 step is 2^-8
+# relative; activations of order 1 pass through a few dozen roundings).
+TOL_BF16 = dict(rtol=2e-2, atol=8e-3)
+
+
+def run_trace(model_dir, dtype, steps, max_tokens):
+    out = tempfile.mkdtemp(prefix="lev_trace_")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype, "--out", out,
+           "--max-tokens", str(max_tokens)]
+    p = subprocess.run(cmd, input=TR.to_jsonl(steps), capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-3000:]
+    assert p.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    return out
+
+
+def read_step(out, step, vocab):
+    return torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_all_cuttings(name, dtype):
+    raw, seed = TINY[name]
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    d = write_model(raw, seed, store)
+    weights = read_weights(d)
+    lengths = [70, 45, 100, 37, 64, 33] if name == "A" else [90, 130, 41, 200, 64, 17]
+    reqs = TR.random_requests(raw["vocab_size"], lengths, seed + 10)
+    rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    plain = {rid: P.plain_logits(weights, raw, torch.tensor(t), rounding=rounding) for rid, t in reqs.items()}
+    steps = TR.number(TR.trace_whole(reqs) + TR.trace_prefill_then_singles(reqs) + TR.trace_portions(reqs)
+                      + TR.trace_mixed(reqs, seed=3) + TR.trace_mixed(reqs, seed=4, prefix="n"))
+    max_tokens = TR.peak_tokens(steps)
+    out = run_trace(d, dtype, steps, max_tokens)
+    want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+    tol = TOL_F32 if dtype == "float32" else TOL_BF16
+    worst = 0.0
+    for s in steps:
+        k = s["step"]
+        assert (k in want) == os.path.exists(os.path.join(out, f"{k}.f32"))
+        if k in want:
+            got = read_step(out, k, raw["vocab_size"])
+            worst = max(worst, float((got.double() - want[k]).abs().max()))
+            torch.testing.assert_close(got.double(), want[k], **tol, msg=lambda m: f"step {k} {s['entries'][0]['id']}: {m}")
+    print(f"trace_run {name} {dtype}: worst abs difference {worst:.3e}")
+    if dtype == "bfloat16":
+        # and against the 32-bit plain implementation: the greedy token agrees wherever its margin is clear
+        plain32 = {rid: P.plain_logits(weights, raw, torch.tensor(t)) for rid, t in reqs.items()}
+        want32 = TR.expected_rows(steps, lambda rid: plain32[rid[1:]])
+        for k, w in want32.items():
+            got = read_step(out, k, raw["vocab_size"])
+            top2 = w.topk(2, dim=-1).values
+            clear = (top2[:, 0] - top2[:, 1]) > 2e-2
+            assert bool((got.argmax(-1)[clear] == w.argmax(-1)[clear]).all())
+            assert float((torch.softmax(got.double(), -1) - torch.softmax(w, -1)).abs().max()) < 1e-2

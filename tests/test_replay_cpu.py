@@ -1,0 +1,102 @@
+"""The step function, the cache manager and the batch tables under every way of cutting the work,
+on the CPU with the emulated kernels: what differs from the plain implementation here is a fault
+of the host logic, not of a kernel."""
+import pytest
+import torch
+
+import plain_gpt2 as P
+import traces as TR
+from emulated_kernels import EmulatedKernels
+from helpers import read_weights, write_model
+from levanter_amd.config import InferenceEngineConfig
+from levanter_amd.engine import ModelRunner, StepEntry, StepError
+from levanter_amd.engine.loading import load_model, make_cache
+from levanter_amd.parts import BuildEnv
+from tiny_configs import TINY
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def setup(request):
+    raw, seed = TINY[request.param]
+    d = write_model(raw, seed, torch.float32)
+    env = BuildEnv(torch.float32, torch.device("cpu"), EmulatedKernels())
+    _, model = load_model(d, env)
+    weights = read_weights(d)
+    lengths = [70, 45, 100, 37, 64, 33] if request.param == "A" else [90, 130, 41, 200, 64, 17]
+    reqs = TR.random_requests(raw["vocab_size"], lengths, seed + 10)
+    plain = {rid: P.plain_logits(weights, raw, torch.tensor(t)) for rid, t in reqs.items()}
+    return raw, model, env, reqs, plain
+
+
+def replay(model, env, steps, max_tokens):
+    ps = 16
+    cfg = InferenceEngineConfig(max_pages=max_tokens // ps, max_seqs=4, page_size=ps, max_pages_per_seq=16, compute_dtype="float32")
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    live, out = {}, {}
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if e["id"] not in live:
+                live[e["id"]] = cache.open(e["id"])
+            entries.append(StepEntry(live[e["id"]], e["tokens"], e["want"]))
+        logits = runner.step(entries)
+        cache.check_invariants()
+        if logits.shape[0]:
+            out[s["step"]] = logits
+        for rid in s["end"]:
+            cache.close(live.pop(rid))
+    cache.check_invariants()
+    assert all(g.pool.n_free == g.pool.n_pages for g in cache.groups)
+    return out
+
+
+@pytest.mark.parametrize("mode", ["whole", "singles", "portions", "mixed"])
+def test_every_way_of_cutting_gives_the_plain_logits(setup, mode):
+    raw, model, env, reqs, plain = setup
+    steps = {"whole": TR.trace_whole, "singles": TR.trace_prefill_then_singles, "portions": TR.trace_portions,
+             "mixed": lambda r: TR.trace_mixed(r, seed=3)}[mode](reqs)
+    TR.number(steps)
+    max_tokens = TR.peak_tokens(steps)
+    got = replay(model, env, steps, max_tokens)
+    want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+    assert set(got) == set(want)
+    for k in want:
+        torch.testing.assert_close(got[k].double(), want[k], rtol=1e-4, atol=1e-5)
+
+
+def test_mixed_trace_really_mixes_and_reuses_pages(setup):
+    raw, model, env, reqs, plain = setup
+    steps = TR.number(TR.trace_mixed(reqs, seed=3))
+    assert any(len(s["entries"]) >= 3 for s in steps)
+    assert any(any(len(e["tokens"]) == 1 for e in s["entries"]) and any(len(e["tokens"]) > 1 for e in s["entries"]) for s in steps)
+    total = sum((len(t) + 63) // 64 * 64 for t in reqs.values())
+    assert TR.peak_tokens(steps) < total  # the pool is smaller than all requests together: pages are used again
+
+
+def test_step_refuses_bad_input(setup):
+    raw, model, env, reqs, plain = setup
+    cfg = InferenceEngineConfig(max_pages=8, max_seqs=2, page_size=16, max_pages_per_seq=32, compute_dtype="float32")
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    h = cache.open("a")
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        runner.step([StepEntry(h, [raw["vocab_size"]], [0])])
+    with pytest.raises(StepError, match="wanted place"):
+        runner.step([StepEntry(h, [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        runner.step([StepEntry(h, [1], []), StepEntry(h, [2], [])])
+    with pytest.raises(StepError, match="no tokens"):
+        runner.step([StepEntry(h, [], [])])
+    with pytest.raises(StepError, match="limit"):  # beyond the position table
+        runner.step([StepEntry(h, [1] * (raw["n_positions"] + 1), [])])
+    assert h.length == 0 and all(g.pool.n_free == 8 for g in cache.groups)  # nothing changed
+    from levanter_amd.cache import OutOfPages
+
+    h2 = cache.open("b")
+    runner.step([StepEntry(h, [1] * 100, [])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry(h2, [1] * 40, [0])])
+    assert h2.length == 0
+    cache.check_invariants()
+    assert runner.step([]).shape == (0, raw["vocab_size"])

@@ -1,0 +1,194 @@
+"""The scheduler's decisions and the engine's bookkeeping, on the CPU: a dummy model with constant
+one-hot logits (as the reference's tests/inference/test_engine.py:19-46), the emulated kernels for
+sampling, and the real cache manager, step function and scheduler."""
+import pytest
+import torch
+
+from emulated_kernels import EmulatedKernels
+from levanter_amd.cache import PagedKv
+from levanter_amd.config import InferenceEngineConfig
+from levanter_amd.engine import InferenceEngine, Request, SeqDecodingParams, is_stop_signal
+from levanter_amd.parts import BuildEnv
+from levanter_amd.parts.spec import PlanEntry
+
+
+class DummyModel:
+    """Keeps pages like a two-layer attention model, computes nothing, prefers token `eos` everywhere
+    (or the token after the input token, with ``count=True``)."""
+
+    def __init__(self, vocab_size=10, eos=3, count=False, max_positions=None):
+        self.vocab_size = vocab_size
+        self.eos = eos
+        self.count = count
+        self.max_positions = max_positions
+        self.plan = [PlanEntry(0, 0), PlanEntry(1, 1)]
+        self.batches = []
+        self.env = None
+
+    def cache_requirements(self):
+        return [(0, PagedKv(1, 16)), (1, PagedKv(1, 16))]
+
+    def forward(self, ctx, rows):
+        self.batches.append(list(ctx.host["run_lengths"]))
+        n = rows.numel()
+        logits = torch.zeros(n, self.vocab_size)
+        if self.count:
+            nxt = (ctx.tokens[rows.long()].long() + 1) % self.vocab_size
+            logits[torch.arange(n), nxt] = 1.0
+        else:
+            logits[:, self.eos] = 1.0
+        return logits
+
+
+def make_engine(model=None, **kw):
+    cfg = InferenceEngineConfig(**{**dict(max_pages=64, max_seqs=8, page_size=16, max_pages_per_seq=4, compute_dtype="float32",
+                                          max_seqs_in_prefill=4), **kw})
+    model = model or DummyModel()
+    env = BuildEnv(torch.float32, torch.device("cpu"), EmulatedKernels())
+    return InferenceEngine(model, cfg, env, allocate=False), model
+
+
+def all_released(engine):
+    engine.cache.check_invariants()
+    return all(int(g.pool.ref_counts.sum()) == 0 for g in engine.cache.groups) and engine.cache.n_free_slots == engine.config.max_seqs
+
+
+def test_release_on_finish_and_reuse_without_reset():
+    # the reference's tests/inference/test_engine.py:62-112: the model always emits 3, which is the stop token
+    engine, _ = make_engine()
+    reqs = [Request(prompt_tokens=p, request_id=i, decode_params=SeqDecodingParams(max_num_tokens=len(p) + 5, stop_tokens=[[3]]))
+            for i, p in enumerate([[7, 7], [1]])]
+    res = engine.generate(reqs)
+    assert res.tokens == [[3], [3]]  # generated tokens only, the stopping token included
+    assert res.finish_reasons == ["stop", "stop"]
+    assert all_released(engine)
+    res = engine.generate(reqs)  # usable again without reset()
+    assert res.tokens == [[3], [3]] and all_released(engine)
+
+
+def test_length_limit_counts_the_prompt():
+    engine, _ = make_engine()
+    r = Request(prompt_tokens=[1, 2, 4], request_id=0, decode_params=SeqDecodingParams(max_num_tokens=7))
+    res = engine.generate([r])
+    assert res.tokens == [[3, 3, 3, 3]] and res.finish_reasons == ["length"] and res.total_generated == 4
+    res = engine.generate([Request(prompt_tokens=[1, 2, 4], request_id=1, max_new_tokens=2)])
+    assert res.tokens == [[3, 3]]
+
+
+def test_stop_sequence_may_begin_in_the_prompt():
+    engine, _ = make_engine(DummyModel(count=True))
+    # counts 5, 6, 7 ...; the stop sequence [4, 5] straddles the end of the prompt
+    res = engine.generate([Request(prompt_tokens=[2, 4], request_id=0, max_new_tokens=6, stop_tokens=[[4, 5]])])
+    assert res.tokens == [[5]]
+    res = engine.generate([Request(prompt_tokens=[2, 4], request_id=0, max_new_tokens=6, stop_tokens=[[9, 9], [6, 7]])])
+    assert res.tokens == [[5, 6, 7]]
+
+
+def test_stop_signal_reference_vectors():
+    # tests/inference/test_inference_utils.py:9-88
+    assert is_stop_signal([5, 6, 7], [[5, 6, 7]])
+    assert not is_stop_signal([5, 6, 7], [[1, 2, 3]])
+    assert is_stop_signal([5, 6, 7], [[6, 7]])
+    assert not is_stop_signal([1, 2, 3], [])
+    assert not is_stop_signal([1, 2, 3], [[]])
+    assert is_stop_signal([8, 9, 10], [[1, 2, 3], [8, 9, 10], [4, 5, 6]])
+    assert not is_stop_signal([28070, 5573, 323, 8254, 1667, 4227, 11, 1057, 2291, 69, 19568, 323, 40317, 743, 704], [[13]])
+
+
+def test_more_requests_than_slots_and_order_of_results():
+    engine, model = make_engine(DummyModel(count=True), max_seqs=2)
+    reqs = [Request(prompt_tokens=[i], request_id=i, max_new_tokens=3) for i in range(5)]
+    res = engine.generate(reqs)
+    assert res.tokens == [[(i + 1) % 10, (i + 2) % 10, (i + 3) % 10] for i in range(5)]
+    assert all_released(engine)
+    assert max(len(b) for b in model.batches) <= 2  # never more than two live sequences
+
+
+def test_prompts_are_cut_under_the_token_budget_and_mixed_with_decoding():
+    engine, model = make_engine(DummyModel(vocab_size=100, count=True), max_prefill_size=7, max_pages_per_seq=8)
+    reqs = [Request(prompt_tokens=list(range(1, 1 + n)), request_id=i, max_new_tokens=4) for i, n in enumerate([3, 20, 9])]
+    res = engine.generate(reqs)
+    assert [len(t) for t in res.tokens] == [4, 4, 4]
+    assert res.tokens[1] == [21, 22, 23, 24]
+    for b in model.batches:  # a step never holds more than 7 prompt tokens
+        assert sum(n for n in b if n > 1) <= 7
+    # some step holds a portion of a prompt beside a single decoded token
+    assert any(1 in b and any(n > 1 for n in b) for b in model.batches)
+    # the 20-token prompt went in as portions
+    assert any(1 < n < 20 for b in model.batches for n in b)
+    assert all_released(engine)
+
+
+def test_pages_run_out_preempts_the_youngest_and_recomputes():
+    # 6 pages of 16 tokens per group; two requests of 40 + 40 tokens need 3 pages each at the end, but a third
+    # one arrives: somebody has to give way, and the tokens equal an unconstrained run
+    big, _ = make_engine(DummyModel(count=True), max_pages=64, max_pages_per_seq=8)
+    small, model = make_engine(DummyModel(count=True), max_pages=6, max_pages_per_seq=8)
+    reqs = [Request(prompt_tokens=[i] * 30, request_id=i, max_new_tokens=30) for i in range(3)]
+    want = big.generate(reqs)
+    got = small.generate(reqs)
+    assert small.scheduler.n_preemptions > 0
+    assert got.tokens == want.tokens
+    assert got.finish_reasons == ["length"] * 3
+    assert all_released(small)
+
+
+def test_a_request_too_large_for_the_pool_fails_alone():
+    engine, _ = make_engine(DummyModel(count=True), max_pages=2, max_pages_per_seq=8)
+    reqs = [Request(prompt_tokens=[1] * 10, request_id=0, max_new_tokens=3),
+            Request(prompt_tokens=[2] * 40, request_id=1, max_new_tokens=3),
+            Request(prompt_tokens=[3] * 10, request_id=2, max_new_tokens=3)]
+    res = engine.generate(reqs)
+    assert res.finish_reasons[0] == "length" and res.finish_reasons[2] == "length"
+    assert res.finish_reasons[1].startswith("error: out of pages")
+    assert res.tokens[0] == [2, 3, 4] and res.tokens[2] == [4, 5, 6]
+    assert all_released(engine)
+
+
+def test_request_validation():
+    engine, _ = make_engine(DummyModel(max_positions=32))
+    with pytest.raises(ValueError, match="empty prompt"):
+        engine.generate([Request(prompt_tokens=[], request_id=0, max_new_tokens=1)])
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        engine.generate([Request(prompt_tokens=[10], request_id=0, max_new_tokens=1)])
+    with pytest.raises(ValueError, match="n_generations"):
+        engine.generate([Request(prompt_tokens=[1], request_id=0, max_new_tokens=1, n_generations=9)])
+    with pytest.raises(ValueError, match="no room"):
+        engine.generate([Request(prompt_tokens=[1] * 32, request_id=0, max_new_tokens=1)])
+    with pytest.raises(ValueError, match="stop sequences"):
+        engine.generate([Request(prompt_tokens=[1], request_id=0, max_new_tokens=1, stop_tokens=[[1]] * 5)])
+    with pytest.raises(ValueError, match="logprobs"):
+        engine.generate([Request(prompt_tokens=[1], request_id=0, max_new_tokens=1, enable_logprobs=True)])
+    # the model's positions bound the length: generation stops at 32 tokens in all
+    res = engine.generate([Request(prompt_tokens=[1] * 30, request_id=0, max_new_tokens=10)])
+    assert len(res.tokens[0]) == 2 and res.finish_reasons == ["length"]
+
+
+def test_n_generations_and_logprobs_and_reset():
+    engine, _ = make_engine(enable_logprobs=True)
+    r = Request(prompt_tokens=[1, 2], request_id=0, max_new_tokens=2, n_generations=3, enable_logprobs=True)
+    res = engine.generate([r])
+    assert res.tokens == [[3, 3]] * 3
+    lp = float(torch.log_softmax(torch.tensor([0.0] * 3 + [1.0] + [0.0] * 6), -1)[3])
+    assert all(abs(x - lp) < 1e-6 for row in res.logprobs for x in row)
+    engine.enqueue_requests([r])
+    engine.step()
+    assert not all_released(engine)
+    engine.reset()
+    assert all_released(engine)
+
+
+def test_temperature_sampling_depends_on_request_and_position_only():
+    # the same request gives the same tokens alone and among others, whatever the budget
+    def run(reqs, **kw):
+        engine, _ = make_engine(DummyModel(vocab_size=50), **kw)
+        return engine.generate(reqs)
+
+    mine = Request(prompt_tokens=[1, 2, 3, 4, 5, 6, 7, 8, 9], request_id=7, max_new_tokens=12, temperature=5.0)
+    alone = run([mine]).tokens[0]
+    others = [Request(prompt_tokens=[4] * n, request_id=i, max_new_tokens=9, temperature=3.0) for i, n in enumerate([1, 20, 5])]
+    mixed = run(others + [mine], max_prefill_size=7).tokens[3]
+    assert alone == mixed
+    assert len(set(alone)) > 3  # it is sampling, not the argmax
+    again = run([Request(prompt_tokens=mine.prompt_tokens, request_id=8, max_new_tokens=12, temperature=5.0)]).tokens[0]
+    assert again != alone  # another request id, another key
