@@ -69,8 +69,8 @@ class InferenceEngine:
                 raise ValueError(f"request {r.request_id}: n_generations={r.n_generations} must be in 1..max_seqs={cfg.max_seqs}")
             if len(r.prompt_tokens) == 0:
                 raise ValueError(f"request {r.request_id}: empty prompt")
-            if len(r.prompt_tokens) >= self.runner.max_len:
-                raise ValueError(f"request {r.request_id}: a prompt of {len(r.prompt_tokens)} tokens leaves no room under the "
+            if len(r.prompt_tokens) > self.runner.max_len:
+                raise ValueError(f"request {r.request_id}: a prompt of {len(r.prompt_tokens)} tokens is longer than the "
                                  f"limit of {self.runner.max_len} (model positions and page_size * max_pages_per_seq)")
             bad = [t for t in r.prompt_tokens if not 0 <= t < v]
             if bad:

@@ -153,8 +153,11 @@ def test_request_validation():
         engine.generate([Request(prompt_tokens=[10], request_id=0, max_new_tokens=1)])
     with pytest.raises(ValueError, match="n_generations"):
         engine.generate([Request(prompt_tokens=[1], request_id=0, max_new_tokens=1, n_generations=9)])
-    with pytest.raises(ValueError, match="no room"):
-        engine.generate([Request(prompt_tokens=[1] * 32, request_id=0, max_new_tokens=1)])
+    with pytest.raises(ValueError, match="longer than the limit"):
+        engine.generate([Request(prompt_tokens=[1] * 33, request_id=0, max_new_tokens=1)])
+    # a prompt that fills the positions exactly still yields the one token its last logits give
+    res = engine.generate([Request(prompt_tokens=[1] * 32, request_id=0, max_new_tokens=5)])
+    assert res.tokens == [[3]] and res.finish_reasons == ["length"]
     with pytest.raises(ValueError, match="stop sequences"):
         engine.generate([Request(prompt_tokens=[1], request_id=0, max_new_tokens=1, stop_tokens=[[1]] * 5)])
     with pytest.raises(ValueError, match="logprobs"):
