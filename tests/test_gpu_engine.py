@@ -1,0 +1,412 @@
+"""The engine on the GPU beyond replay: each part alone against its plain function, long decoding,
+the first tokens of a sequence, generation through the entry point (greedy and sampled), and the
+generality of the parts: a window, a layer named twice, a layer that reads another layer's cache,
+and a toy mixer with state of its own that is registered here, without a change to the framework."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import plain_gpt2 as P
+from emulated_kernels import gumbel_noise
+from helpers import make_meta, read_weights, write_model
+from tiny_configs import TINY, TINY_A, TINY_B
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _env(dtype):
+    from levanter_amd.engine.loading import make_env
+
+    return make_env(dtype)
+
+
+def _ctx(env, tokens, runs):
+    """A StepContext without a cache, for parts that need none."""
+    from levanter_amd.parts import StepContext
+
+    t = torch.tensor(tokens, dtype=torch.int32, device=DEV)
+    return StepContext(kernels=env.kernels, dtype=env.dtype, device=env.device, n_tokens=len(tokens), tokens=t,
+                       attention=make_meta(runs, DEV), seq_slots=torch.zeros(len(runs), dtype=torch.int32, device=DEV),
+                       host={"run_lengths": [q for q, _ in runs], "first_positions": [k - q for q, k in runs], "slots": [0] * len(runs)})
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_each_part_alone(name, dtype):
+    from levanter_amd.config import InferenceEngineConfig, LmConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import load_model, make_cache
+
+    raw, seed = TINY[name]
+    d = write_model(raw, seed, torch.float32 if dtype == "float32" else torch.bfloat16)
+    w = read_weights(d)
+    env = _env(dtype)
+    _, model = load_model(d, env)
+    s = P.plain_sizes(raw)
+    rnd = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == "float32" else dict(rtol=2e-2, atol=2e-3)
+    T = 23
+    g = torch.Generator().manual_seed(1)
+    toks = torch.randint(0, s["V"], (T,), generator=g)
+    ctx = _ctx(env, toks.tolist(), [(T, T)])
+    # embedding with the position encoding
+    x = model.embedding(ctx)
+    want_x = P.plain_embed(toks, torch.arange(T), w["wte.weight"], w["wpe.weight"])
+    torch.testing.assert_close(x.cpu().double(), want_x, rtol=1e-6, atol=1e-7)
+    # a shifted portion uses absolute positions
+    ctx5 = _ctx(env, toks[5:].tolist(), [(T - 5, T)])
+    torch.testing.assert_close(model.embedding(ctx5).cpu().double(), want_x[5:], rtol=1e-6, atol=1e-7)
+    blk = model.blocks[1]
+    # norm
+    xin = (torch.randn(T, s["D"], generator=g) * 2 + 0.5)
+    h = blk.norm1(xin.to(DEV), ctx)
+    want_h = rnd(P.plain_layernorm(xin.double(), w["h.1.ln_1.weight"], w["h.1.ln_1.bias"], raw["layer_norm_epsilon"]))
+    torch.testing.assert_close(h.cpu().double(), want_h, **tol)
+    # feed-forward (adds to the residual in place)
+    hin = rnd(torch.randn(T, s["D"], generator=g).double())
+    res = torch.randn(T, s["D"], generator=g)
+    xr = res.to(DEV).clone()
+    blk.feed_forward.forward(hin.to(env.dtype).to(DEV), xr, ctx)
+    want = res.double() + P.plain_mlp(hin, w, "h.1.", raw, rnd)
+    torch.testing.assert_close(xr.cpu().double(), want, **tol)
+    # head on gathered rows
+    rows = torch.tensor([T - 1, 3], dtype=torch.int32, device=DEV)
+    hf = model.final_norm(xin.to(DEV), ctx, rows=rows)
+    logits = model.head(hf, ctx)
+    want_hf = rnd(P.plain_layernorm(xin.double()[[T - 1, 3]], w["ln_f.weight"], w["ln_f.bias"], raw["layer_norm_epsilon"]))
+    torch.testing.assert_close(logits.cpu().double(), want_hf @ w["wte.weight"].T, **tol)
+    # the mixer, through a cache of its own: a whole sequence, then the same cut in two portions
+    cfg = InferenceEngineConfig(max_pages=8, max_seqs=2, page_size=16, max_pages_per_seq=4, compute_dtype=dtype)
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    want_a = P.plain_attention_layer(hin, w, "h.1.", raw, 1, rnd)
+    for cuts in ([T], [9, T - 9]):
+        hnd = cache.open("x")
+        got = []
+        i = 0
+        for n in cuts:
+            cache.extend(hnd, n)
+            mctx = _ctx(env, toks[i:i + n].tolist(), [(n, i + n)])
+            from levanter_amd.parts import CacheUnitView, GroupView
+
+            grp = cache.groups[0]
+            bt = torch.tensor(grp.block_tables[[hnd.slot], :4], device=DEV)
+            dest = torch.tensor([cache.destination(grp, hnd, p) for p in range(i, i + n)], dtype=torch.int32, device=DEV)
+            k_pages, v_pages, _ = cache.unit_pages(1)
+            unit = CacheUnitView(k_pages=k_pages, v_pages=v_pages, group=GroupView(16, bt, dest))
+            xz = torch.zeros(n, s["D"], device=DEV)
+            blk.mixer.forward(hin[i:i + n].to(env.dtype).to(DEV), xz, mctx, unit, True)
+            got.append(xz.cpu().double())
+            cache.advance(hnd, n)
+            i += n
+        torch.testing.assert_close(torch.cat(got), want_a, **tol)
+        cache.close(hnd)
+
+
+def _engine(d, dtype, **kw):
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import InferenceEngine
+
+    cfg = InferenceEngineConfig(**{**dict(max_seqs=4, page_size=16, max_pages_per_seq=16, compute_dtype=dtype), **kw})
+    return InferenceEngine.from_pretrained(d, cfg)
+
+
+def _check_greedy(weights, raw, prompt, generated, rounding=lambda x: x, margin=1e-4):
+    """Every generated token is the plain implementation's argmax after the tokens before it (where the
+    plain top two are further apart than ``margin``)."""
+    toks = list(prompt) + list(generated)
+    logits = P.plain_logits(weights, raw, torch.tensor(toks), rounding=rounding)
+    n_clear = 0
+    for i, tok in enumerate(generated):
+        row = logits[len(prompt) - 1 + i]
+        top = row.topk(2).values
+        if float(top[0] - top[1]) > margin:
+            n_clear += 1
+            assert int(row.argmax()) == tok, f"generated token {i}"
+    return n_clear
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(dtype):
+    # the workload of tiny configuration A: prompts of 5, 17 and 33 tokens, 16 greedy tokens each
+    from levanter_amd.engine import Request
+
+    d = write_model(TINY_A, 0, torch.float32 if dtype == "float32" else torch.bfloat16)
+    w = read_weights(d)
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist() for n in (5, 17, 33)]
+    engine = _engine(d, dtype)
+    res = engine.generate([Request(prompt_tokens=p, request_id=i, max_new_tokens=16) for i, p in enumerate(prompts)])
+    assert [len(t) for t in res.tokens] == [16, 16, 16] and res.finish_reasons == ["length"] * 3
+    if dtype == "float32":
+        for p, out in zip(prompts, res.tokens):
+            assert out == P.plain_greedy_generate(w, TINY_A, p, 16)
+    else:
+        clear = sum(_check_greedy(w, TINY_A, p, out, P.bf16_rounding, margin=2e-2) for p, out in zip(prompts, res.tokens))
+        assert clear >= 10
+    engine.cache.check_invariants()
+    assert engine.cache.n_free_slots == 4
+
+
+def test_sampled_generation_mixed_batch_fixed_seed():
+    # the workload of tiny configuration B: prompts of 1, 9, 40 and 100 tokens, prefilled in portions of 7
+    # beside decoding requests, then 24 steps at temperature 0.8 with a fixed seed. Every sampled token is
+    # argmax(plain logits / T + the documented noise of (request key, position)).
+    from levanter_amd.engine import Request
+
+    d = write_model(TINY_B, 1, torch.float32)
+    w = read_weights(d)
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (1, 9, 40, 100)]
+    engine = _engine(d, "float32", max_prefill_size=7, seed=5, enable_logprobs=True)
+    reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=24, temperature=0.8, enable_logprobs=True) for i, p in enumerate(prompts)]
+    seqs = engine.enqueue_requests(reqs)
+    while not all(s.done for s in seqs):
+        engine.step()
+    for s in seqs:
+        toks = s.tokens
+        logits = P.plain_logits(w, TINY_B, torch.tensor(toks))
+        for i, tok in enumerate(s.generated):
+            pos = s.request.prompt_tokens.__len__() - 1 + i
+            scaled = logits[pos].float() / 0.8
+            noisy = scaled + gumbel_noise(s.key[0], s.key[1], pos, 1000)
+            top = noisy.topk(2).values
+            if float(top[0] - top[1]) > 1e-3:
+                assert int(noisy.argmax()) == tok
+            assert abs(s.logprobs[i] - float(torch.log_softmax(scaled, -1)[tok])) < 1e-3
+    # alone, the longest request gives the same tokens: sampling does not depend on the batch
+    alone = _engine(d, "float32", seed=5, enable_logprobs=True).generate([reqs[3]]).tokens[0]
+    assert alone == seqs[3].generated
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(dtype):
+    from levanter_amd.engine import Request
+
+    d = write_model(TINY_B, 1, torch.float32 if dtype == "float32" else torch.bfloat16)
+    w = read_weights(d)
+    # sharpen attention so that a wrong or stale key would change the argmax: scale the q and k columns
+    # of every layer (the file is rewritten; the plain implementation reads the same file)
+    from levanter_amd.weights import save_file
+    from safetensors.torch import load_file
+    import os
+
+    t = load_file(os.path.join(d, "model.safetensors"))
+    for i in range(3):
+        t[f"h.{i}.attn.c_attn.weight"][:, :192] *= 12.0
+    save_file(t, os.path.join(d, "model.safetensors"))
+    w = read_weights(d)
+    engine = _engine(d, dtype, max_pages=40)
+    rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    margin = 1e-4 if dtype == "float32" else 3e-2
+    # one prompt token, then 250 decoded tokens up to the end of the position table (256)
+    res = engine.generate([Request(prompt_tokens=[7], request_id=0, max_new_tokens=400)])
+    out = res.tokens[0]
+    assert len(out) == 255 and res.finish_reasons == ["length"]
+    assert _check_greedy(w, TINY_B, [7], out, rounding, margin) >= (250 if dtype == "float32" else 100)
+    # the first tokens: sequences of one, two and three tokens in one batch
+    res = engine.generate([Request(prompt_tokens=[5], request_id=1, max_new_tokens=3),
+                           Request(prompt_tokens=[9, 4], request_id=2, max_new_tokens=2),
+                           Request(prompt_tokens=[1, 2, 3], request_id=3, max_new_tokens=1)])
+    for p, o in zip(([5], [9, 4], [1, 2, 3]), res.tokens):
+        _check_greedy(w, TINY_B, p, o, rounding, margin)
+
+
+# ------------------------------------------------------------------------------------------------
+# Generality of the parts, shown with toy architectures that exist only in this test.
+
+def _toy_spec(window=None, plan=None, n_layer=2, mixers=None):
+    """A two-layer GPT-2-like description over tiny A's tensors, with options GPT-2 itself does not have."""
+    from levanter_amd.config import LmConfig
+    from levanter_amd.parts.spec import PlanEntry
+
+    spec = LmConfig.from_dict(dict(TINY_A, n_layer=n_layer)).model_spec()
+    for i, layer in enumerate(spec.layers):
+        if window is not None and i == 1:
+            layer.mixer.params["window"] = window
+        if mixers and mixers[i] is not None:
+            layer.mixer = mixers[i]
+    if plan is not None:
+        spec.plan = [PlanEntry(*p) for p in plan]
+    return spec
+
+
+def _run_cut(spec, tensors, dtype, toks, cuts, n_pages=16, state_checks=None):
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import make_cache
+    from levanter_amd.parts import DecoderLm
+
+    env = _env(dtype)
+    model = DecoderLm(spec, tensors, env)
+    cfg = InferenceEngineConfig(max_pages=n_pages, max_seqs=2, page_size=16, max_pages_per_seq=8, compute_dtype=dtype)
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    h = cache.open("t")
+    out, i = [], 0
+    for n in cuts:
+        out.append(runner.step([StepEntry(h, toks[i:i + n], list(range(n)))]).cpu())
+        cache.check_invariants()
+        i += n
+    return torch.cat(out), cache, h
+
+
+def test_window_layer_has_its_own_pages_and_gives_them_back():
+    d = write_model(TINY_A, 0, torch.float32)
+    w = read_weights(d)
+    t32 = {k: v.float() for k, v in w.items()}
+    W = 20
+    spec = _toy_spec(window=W)
+    toks = torch.randint(0, 512, (100,), generator=torch.Generator().manual_seed(3)).tolist()
+    # plain: layer 0 sees everything, layer 1 a window of 20 keys
+    x = P.plain_embed(torch.tensor(toks), torch.arange(100), w["wte.weight"], w["wpe.weight"])
+    for i in range(2):
+        p = f"h.{i}."
+        hh = P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5)
+        q, k, v = P.plain_split_qkv(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"]), 4)
+        o = P.plain_causal_attention(q, k, v, window=W if i == 1 else None)
+        x = x + P.plain_linear(o.transpose(0, 1).reshape(100, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+        x = x + P.plain_mlp(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5), w, p, TINY_A)
+    want = P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+    for cuts in ([100], [37, 2, 30, 1, 1, 1, 28], [1] * 100):
+        got, cache, h = _run_cut(spec, t32, "float32", toks, cuts, n_pages=7)
+        torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-5)
+        assert len(cache.groups) == 2
+        g_all, g_win = cache.groups if cache.groups[0].requirement.window is None else cache.groups[::-1]
+        assert len(g_all.pages_held(h.slot)) == 7 and len(g_win.pages_held(h.slot)) <= 3
+
+
+def test_a_layer_named_twice_and_a_layer_reading_anothers_cache():
+    d = write_model(TINY_A, 0, torch.float32)
+    w = read_weights(d)
+    t32 = {k: v.float() for k, v in w.items()}
+    toks = torch.randint(0, 512, (40,), generator=torch.Generator().manual_seed(4)).tolist()
+
+    def plain(order):
+        x = P.plain_embed(torch.tensor(toks), torch.arange(40), w["wte.weight"], w["wpe.weight"])
+        kv = {}
+        for layer, unit, writes in order:
+            p = f"h.{layer}."
+            hh = P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5)
+            q, k, v = P.plain_split_qkv(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"]), 4)
+            if writes:
+                kv[unit] = (k, v)
+            k, v = kv[unit]
+            o = P.plain_causal_attention(q, k, v)
+            x = x + P.plain_linear(o.transpose(0, 1).reshape(40, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+            x = x + P.plain_mlp(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5), w, p, TINY_A)
+        return P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+
+    # layer 0 runs twice (two cache units of its own), then layer 1 reads the keys and values that the
+    # first run of layer 0 wrote (unit 0) instead of writing its own
+    order = [(0, 0, True), (0, 1, True), (1, 0, False)]
+    want = plain(order)
+    for cuts in ([40], [13, 2, 24, 1]):
+        got, cache, _ = _run_cut(_toy_spec(plan=order), t32, "float32", toks, cuts)
+        torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-5)
+        assert sorted(u for g in cache.groups for u in g.units) == [0, 1]
+    from levanter_amd.parts import DecoderLm
+
+    with pytest.raises(ValueError, match="before any entry has written"):
+        DecoderLm(_toy_spec(plan=[(0, 0, False), (1, 1, True)]), t32, _env("float32"))
+
+
+def test_a_toy_mixer_with_state_of_its_own_registers_builds_and_steps():
+    """A mixer defined here: the running mean of its inputs over the request so far, kept as a sum and a
+    count in a per-request slot. Registered, built from a description and stepped in portions, with the
+    attention layer beside it, without touching the framework's files."""
+    from levanter_amd.cache import SlotState
+    from levanter_amd.parts import MIXERS, Mixer, PartSpec
+
+    D = 64
+
+    @MIXERS.register("toy_running_mean")
+    class RunningMean(Mixer):
+        def __init__(self, spec, tensors, env):
+            super().__init__(spec, tensors, env)
+            self.gain = float(spec.params["gain"])
+
+        def cache_requirement(self):
+            return SlotState((D + 1,), "float32")
+
+        def forward(self, h, x, ctx, unit, writes_cache):
+            t0 = 0
+            for n, slot in zip(ctx.host["run_lengths"], ctx.host["slots"]):
+                st = unit.state[slot]
+                run = h[t0:t0 + n].float()
+                sums = st[:D] + torch.cumsum(run, 0)
+                counts = st[D] + torch.arange(1, n + 1, device=h.device, dtype=torch.float32)
+                x[t0:t0 + n] += self.gain * sums / counts[:, None]
+                st[:D] = sums[-1]
+                st[D] = counts[-1]
+                t0 += n
+
+    try:
+        d = write_model(TINY_A, 0, torch.float32)
+        w = read_weights(d)
+        t32 = {k: v.float() for k, v in w.items()}
+        spec = _toy_spec(mixers=[None, PartSpec("toy_running_mean", {"gain": 0.5}, {})])
+        toks = torch.randint(0, 512, (50,), generator=torch.Generator().manual_seed(6)).tolist()
+        x = P.plain_embed(torch.tensor(toks), torch.arange(50), w["wte.weight"], w["wpe.weight"])
+        x = P.plain_block(x, w, TINY_A, 0)
+        hh = P.plain_layernorm(x, w["h.1.ln_1.weight"], w["h.1.ln_1.bias"], 1e-5)
+        x = x + 0.5 * torch.cumsum(hh, 0) / torch.arange(1, 51).unsqueeze(1)
+        x = x + P.plain_mlp(P.plain_layernorm(x, w["h.1.ln_2.weight"], w["h.1.ln_2.bias"], 1e-5), w, "h.1.", TINY_A)
+        want = P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+        for cuts in ([50], [20, 2, 27, 1]):
+            got, cache, h = _run_cut(spec, t32, "float32", toks, cuts)
+            torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-4)
+            assert list(cache.state.tensors) == [1] and float(cache.state.tensors[1][h.slot, D]) == 50.0
+            cache.close(h)
+            h2 = cache.open("again")  # the slot is zeroed for the next request
+            assert h2.slot == h.slot and float(cache.state.tensors[1][h2.slot].abs().sum()) == 0.0
+    finally:
+        MIXERS.unregister("toy_running_mean")
+
+
+def test_a_new_architecture_registers_without_touching_the_framework(tmp_path):
+    """A configuration class and description registered under a new model_type: the folder's config.json
+    picks it, the loader checks its tensors, the engine runs it."""
+    import json
+
+    from levanter_amd.config import LmConfig
+    from levanter_amd.engine import InferenceEngine, Request
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.weights import write_random_model
+
+    @LmConfig.register_subclass("toy_gpt_rms")
+    @dataclass(frozen=True)
+    class ToyConfig(LmConfig):
+        vocab_size: int = 300
+        dim: int = 48
+        heads: int = 3
+        layers: int = 2
+
+        @classmethod
+        def from_hf_config(cls, raw):
+            return cls(**{k: raw[k] for k in ("vocab_size", "dim", "heads", "layers") if k in raw})
+
+        def to_hf_config(self):
+            return {"model_type": "toy_gpt_rms", "vocab_size": self.vocab_size, "dim": self.dim, "heads": self.heads, "layers": self.layers}
+
+        def model_spec(self):
+            from levanter_amd.config import Gpt2Config
+
+            spec = Gpt2Config(vocab_size=self.vocab_size, n_positions=64, n_embd=self.dim, n_layer=self.layers, n_head=self.heads).model_spec()
+            spec.architecture = "toy_gpt_rms"
+            for layer in spec.layers:
+                layer.norm1.kind = layer.norm2.kind = "rmsnorm"
+            spec.final_norm.kind = "rmsnorm"
+            return spec
+
+    try:
+        write_random_model(ToyConfig(), 3, str(tmp_path))
+        assert json.load(open(tmp_path / "config.json"))["model_type"] == "toy_gpt_rms"
+        engine = InferenceEngine.from_pretrained(str(tmp_path), InferenceEngineConfig(max_seqs=2, max_pages_per_seq=4, compute_dtype="float32"))
+        res = engine.generate([Request(prompt_tokens=[1, 2, 3], request_id=0, max_new_tokens=5)])
+        assert len(res.tokens[0]) == 5
+    finally:
+        LmConfig.unregister("toy_gpt_rms")
