@@ -3,17 +3,33 @@
 
 // ------------------------------------------------------------------------------------------
 // x[t, :] = float(table[token_t, :]) + float(pos_table[pos_t, :])        (32-bit residual stream)
+// Several rows per block when rows are short; 4 elements per thread and iteration so that a row's
+// loads are in flight together (a single block is bound by memory latency, not by bandwidth).
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
-                             const T* __restrict__ table, const T* __restrict__ pos_table, float* __restrict__ out, int D) {
+__global__ void __launch_bounds__(256)
+embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions, const T* __restrict__ table,
+             const T* __restrict__ pos_table, float* __restrict__ out, int D) {
   const int t = blockIdx.x;
   const T* row = table + (size_t)tokens[t] * D;
   const T* prow = pos_table ? pos_table + (size_t)positions[t] * D : nullptr;
   float* o = out + (size_t)t * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float v = to_float<T>(row[d]);
-    if (prow) v += to_float<T>(prow[d]);
-    o[d] = v;
+  if ((D & 3) == 0) {
+    for (int d = threadIdx.x * 4; d < D; d += 1024) {
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = to_float<T>(row[d + j]);
+      if (prow) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += to_float<T>(prow[d + j]);
+      }
+      *reinterpret_cast<float4*>(o + d) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += 256) {
+      float v = to_float<T>(row[d]);
+      if (prow) v += to_float<T>(prow[d]);
+      o[d] = v;
+    }
   }
 }
 
@@ -32,6 +48,67 @@ extern "C" int lev_embed(const int* tokens, const int* positions, const void* ta
 // ------------------------------------------------------------------------------------------
 // One block per output row. Statistics in 32-bit, two passes (mean, then the centred squares).
 // rows != null: output row r is the norm of input row rows[r] (the wanted rows before the head).
+// Rows of up to NT * 4 * NV floats are read once, as float4, into registers: every load of the row is in
+// flight at the same time. Longer rows (or a width that is no multiple of 4) take the looping kernel.
+template <typename TO>
+__device__ __forceinline__ void store4(TO* p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
+  uint2 v;
+  v.x = (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
+  v.y = (uint32_t)float_to_bf16(c) | ((uint32_t)float_to_bf16(d) << 16);
+  *reinterpret_cast<uint2*>(p) = v;
+}
+
+template <typename TO, int NT, int NV>
+__global__ void __launch_bounds__(NT)
+norm_reg_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ out,
+                const int* __restrict__ rows, int D, float eps, int rms) {
+  __shared__ float red[NT / 64];
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * D;
+  float4 v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int d = (threadIdx.x + i * NT) * 4;
+    v[i] = d < D ? *reinterpret_cast<const float4*>(xr + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float mean = 0.f;
+  if (!rms) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    mean = block_sum<NT>(s, red) / (float)D;
+  }
+  float s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int d = (threadIdx.x + i * NT) * 4;
+    if (d < D) {
+      const float c0 = v[i].x - mean, c1 = v[i].y - mean, c2 = v[i].z - mean, c3 = v[i].w - mean;
+      s2 += (c0 * c0 + c1 * c1) + (c2 * c2 + c3 * c3);
+    }
+  }
+  const float var = block_sum<NT>(s2, red) / (float)D;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  TO* o = out + (size_t)r * D;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int d = (threadIdx.x + i * NT) * 4;
+    if (d < D) {
+      const float4 wv = *reinterpret_cast<const float4*>(w + d);
+      float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (b) bv = *reinterpret_cast<const float4*>(b + d);
+      store4<TO>(o + d, (v[i].x - mean) * rstd * wv.x + bv.x, (v[i].y - mean) * rstd * wv.y + bv.y,
+                 (v[i].z - mean) * rstd * wv.z + bv.z, (v[i].w - mean) * rstd * wv.w + bv.w);
+    }
+  }
+}
+
 template <typename TO, int NT>
 __global__ void norm_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b,
                             TO* __restrict__ out, const int* __restrict__ rows, int D, float eps, int rms) {
@@ -59,6 +136,17 @@ __global__ void norm_kernel(const float* __restrict__ x, const float* __restrict
   }
 }
 
+template <typename TO>
+static void launch_norm(const float* x, const float* w, const float* b, TO* out, const int* rows, int n_rows, int D, float eps,
+                        int rms, hipStream_t stream) {
+  if ((D & 3) == 0 && D <= 256 * 4 * 2)
+    norm_reg_kernel<TO, 256, 2><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+  else if ((D & 3) == 0 && D <= 256 * 4 * 8)
+    norm_reg_kernel<TO, 256, 8><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+  else
+    norm_kernel<TO, 256><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+}
+
 extern "C" int lev_norm(const float* x, const float* w, const float* b, void* out, const int* rows, int n_rows, int D,
                         float eps, int rms, int out_dtype, hipStream_t stream) {
   LEV_REQUIRE(n_rows >= 0 && D > 0, "norm: bad sizes rows=%d D=%d", n_rows, D);
@@ -66,9 +154,9 @@ extern "C" int lev_norm(const float* x, const float* w, const float* b, void* ou
   LEV_REQUIRE(eps > 0.f, "norm: eps must be positive");
   if (n_rows == 0) return 0;
   if (out_dtype == LEV_F32)
-    norm_kernel<float, 256><<<n_rows, 256, 0, stream>>>(x, w, b, (float*)out, rows, D, eps, rms);
+    launch_norm<float>(x, w, b, (float*)out, rows, n_rows, D, eps, rms, stream);
   else
-    norm_kernel<bf16_t, 256><<<n_rows, 256, 0, stream>>>(x, w, b, (bf16_t*)out, rows, D, eps, rms);
+    launch_norm<bf16_t>(x, w, b, (bf16_t*)out, rows, n_rows, D, eps, rms, stream);
   return lev_check_launch("norm");
 }
 

@@ -150,7 +150,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int nsteps = (K + 31) / 32;
-  constexpr int U = 4;  // k-steps whose loads are issued together
+  constexpr int U = MT == 1 ? 8 : 4;  // k-steps whose loads are issued together (bytes in flight per wave)
   for (int s0 = wave; s0 < nsteps; s0 += WAVES * U) {
     u32x4 wv[U];
     u32x4 av[U][MT];

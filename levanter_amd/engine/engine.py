@@ -106,7 +106,7 @@ class InferenceEngine:
             return []
         entries = [StepEntry(e.seq.handle, e.tokens, [len(e.tokens) - 1] if e.wants_logits else []) for e in plan]
         t0 = time.perf_counter()
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, copy_out=False)
         wanted = [e for e in plan if e.wants_logits]
         toks: List[int] = []
         lps: List[float] = []
@@ -114,9 +114,7 @@ class InferenceEngine:
             temps = [e.seq.request.decode_params.temperature for e in wanted]
             keys = [e.seq.key for e in wanted]
             positions = [e.seq.n_cached - 1 for e in wanted]  # position of the token whose logits are sampled
-            t, lp = self.sampler(logits, temps, keys, positions)
-            toks = t.cpu().tolist()
-            lps = lp.cpu().tolist()
+            toks, lps = self.sampler.to_host(logits, temps, keys, positions)
         self.stats["steps"] += 1
         self.stats["tokens_in"] += sum(len(e.tokens) for e in plan)
         self.stats["device_s"] += time.perf_counter() - t0

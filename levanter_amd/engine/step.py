@@ -41,13 +41,15 @@ class StepError(ValueError):
 class ModelRunner:
     """Owns the model, the cache manager's device tensors and the step function."""
 
-    def __init__(self, model: DecoderLm, cache: CacheManager, env: BuildEnv, allocate: bool = True):
+    def __init__(self, model: DecoderLm, cache: CacheManager, env: BuildEnv, allocate: bool = True, use_graphs: bool = True):
         self.model = model
         self.cache = cache
         self.env = env
         if allocate:
             cache.allocate_tensors(env.dtype, env.device)
         self._workspaces: Dict[object, torch.Tensor] = {}
+        self._graphs: Dict[tuple, object] = {}
+        self.use_graphs = bool(use_graphs) and env.device.type == "cuda" and getattr(model, "graph_safe", False)
         limit = cache.page_size * cache.max_pages_per_seq
         mp = model.max_positions
         self.max_len = limit if mp is None else min(limit, mp)
@@ -85,9 +87,10 @@ class ModelRunner:
                     raise StepError(f"request {rid!r}: wanted place {w} is not among its {n} tokens")
 
     # ------------------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], copy_out: bool = True) -> torch.Tensor:
         """Run the entries as one batch. Returns float32 logits [wanted, vocab] in the order of the
-        entries and of their ``want``. Raises ``OutOfPages`` (nothing changed) if a pool is too small."""
+        entries and of their ``want``. Raises ``OutOfPages`` (nothing changed) if a pool is too small.
+        ``copy_out=False`` may return a buffer that the next step overwrites (the sampler reads it at once)."""
         entries = list(entries)
         self._validate(entries)
         if not entries:
@@ -98,7 +101,22 @@ class ModelRunner:
                 f"{n} of group {g.index}'s {g.pool.n_free} free" for n, g in zip(need, self.cache.groups)))
         for e in entries:
             self.cache.extend(e.handle, len(e.tokens))
+        graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+        batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1)
+        if graphable:
+            logits = self._run_graphed(batch)
+            if copy_out:
+                logits = logits.clone()
+        else:
+            logits = self.model.forward(self._make_ctx(self._upload(batch.host), batch, self._workspaces), batch.rows_view)
+        for e in entries:
+            self.cache.advance(e.handle, len(e.tokens))
+        return logits
 
+    # ------------------------------------------------------------------------------------
+    def _build_host(self, entries: Sequence[StepEntry], pad_blocks: int = 1) -> "HostBatch":
+        """Everything the GPU needs to know about the step, in one int32 buffer with a layout that
+        depends only on (tokens, requests, wanted rows, tiles, single tokens, blocks per request)."""
         cache, ps = self.cache, self.cache.page_size
         S = len(entries)
         T = sum(len(e.tokens) for e in entries)
@@ -110,7 +128,7 @@ class ModelRunner:
         tiles: List[int] = []
         decode: List[int] = []
         run_lengths, first_positions = [], []
-        max_blocks, max_kv = 1, 1
+        max_blocks = 1
         t0 = 0
         for s, e in enumerate(entries):
             n, start = len(e.tokens), e.handle.length
@@ -127,11 +145,10 @@ class ModelRunner:
             run_lengths.append(n)
             first_positions.append(start)
             max_blocks = max(max_blocks, (start + n + ps - 1) // ps)
-            max_kv = max(max_kv, start + n)
             t0 += n
-
+        if pad_blocks > 1:
+            max_blocks = min((max_blocks + pad_blocks - 1) // pad_blocks * pad_blocks, cache.max_pages_per_seq)
         n_groups = len(cache.groups)
-        # one int32 buffer for everything that goes to the GPU
         sizes = [T, T, T, S, len(rows), len(tiles), len(decode)] + [S * max_blocks, T] * n_groups
         offs = np.concatenate([[0], np.cumsum([(x + 3) // 4 * 4 for x in sizes])]).astype(np.int64)
         host = np.zeros(int(offs[-1]), np.int32)
@@ -140,32 +157,28 @@ class ModelRunner:
         for gi, g in enumerate(cache.groups):
             bt = g.block_tables[seq_slots, :max_blocks]
             host[offs[7 + 2 * gi]:offs[7 + 2 * gi] + S * max_blocks] = bt.reshape(-1)
-            dest = np.empty(T, np.int32)
-            t0 = 0
-            for s, e in enumerate(entries):
-                n, start = len(e.tokens), e.handle.length
-                pos = np.arange(start, start + n)
-                pages = g.block_tables[e.handle.slot, pos // ps]
-                assert (pages != NO_PAGE).all(), "a new token has no page"
-                dest[t0:t0 + n] = pages * ps + pos % ps
-                t0 += n
-            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = dest
-        dev = self._upload(host)
+            pages = g.block_tables[seq_slots[token_seq], positions // ps]
+            assert (pages != NO_PAGE).all(), "a new token has no page"
+            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = pages * ps + positions % ps
+        return HostBatch(host=host, sizes=sizes, offs=[int(o) for o in offs], n_tokens=T, n_seqs=S, n_rows=len(rows),
+                         n_tiles=len(tiles) // 2, n_decode=len(decode), max_blocks=max_blocks, max_kv=max_blocks * ps,
+                         run_lengths=run_lengths, first_positions=first_positions, slots=[int(x) for x in seq_slots])
 
+    def _make_ctx(self, dev: torch.Tensor, b: "HostBatch", workspaces: Dict[object, torch.Tensor]) -> StepContext:
         def view(i):
-            return dev[int(offs[i]):int(offs[i]) + sizes[i]]
+            return dev[b.offs[i]:b.offs[i] + b.sizes[i]]
 
+        cache, ps = self.cache, self.cache.page_size
         meta = AttentionMeta(
             positions=view(1), token_seq=view(2),
-            prefill_tiles=view(5).view(-1, 2) if tiles else None, n_prefill_tiles=len(tiles) // 2,
-            decode_tokens=view(6) if decode else None, n_decode=len(decode),
-            max_kv_len=max_kv, _workspaces=self._workspaces)
-        ctx = StepContext(kernels=self.env.kernels, dtype=self.env.dtype, device=self.env.device, n_tokens=T, tokens=view(0),
-                          attention=meta, seq_slots=view(3),
-                          host={"run_lengths": run_lengths, "first_positions": first_positions,
-                                "slots": [int(s) for s in seq_slots]})
-        group_views = [GroupView(page_size=ps, block_tables=view(7 + 2 * gi).view(S, max_blocks), dest=view(8 + 2 * gi))
-                       for gi in range(n_groups)]
+            prefill_tiles=view(5).view(-1, 2) if b.n_tiles else None, n_prefill_tiles=b.n_tiles,
+            decode_tokens=view(6) if b.n_decode else None, n_decode=b.n_decode,
+            max_kv_len=b.max_kv, _workspaces=workspaces)
+        ctx = StepContext(kernels=self.env.kernels, dtype=self.env.dtype, device=self.env.device, n_tokens=b.n_tokens,
+                          tokens=view(0), attention=meta, seq_slots=view(3),
+                          host={"run_lengths": b.run_lengths, "first_positions": b.first_positions, "slots": b.slots})
+        group_views = [GroupView(page_size=ps, block_tables=view(7 + 2 * gi).view(b.n_seqs, b.max_blocks), dest=view(8 + 2 * gi))
+                       for gi in range(len(cache.groups))]
         for unit, g in cache.group_of_unit.items():
             i = g.unit_pos[unit]
             ctx.units[unit] = CacheUnitView(k_pages=None if g.k_pages is None else g.k_pages[i],
@@ -174,14 +187,74 @@ class ModelRunner:
             ctx.units[unit] = CacheUnitView(state=t)
         for e in self.model.plan:  # units whose mixers keep nothing still need a view
             ctx.units.setdefault(e.cache, CacheUnitView())
-
-        logits = self.model.forward(ctx, view(4))
-        for e in entries:
-            cache.advance(e.handle, len(e.tokens))
-        return logits
+        b.rows_view = view(4)
+        return ctx
 
     def _upload(self, host: np.ndarray) -> torch.Tensor:
         t = torch.from_numpy(host)
         if self.env.device.type == "cpu":
             return t
         return t.pin_memory().to(self.env.device, non_blocking=True)
+
+    # ---- decode steps as HIP graphs --------------------------------------------------------
+    def _run_graphed(self, b: "HostBatch") -> torch.Tensor:
+        """A step of single tokens has a kernel sequence that depends only on (requests, wanted rows,
+        blocks per request): the second time such a step comes it is captured into a HIP graph whose
+        inputs live in a fixed device buffer; later steps copy their tables there and replay it."""
+        key = (b.n_seqs, b.n_rows, b.max_blocks)
+        entry = self._graphs.get(key)
+        if entry is None:  # first time: run eagerly (also loads every kernel the graph will need)
+            self._graphs[key] = "seen"
+            return self.model.forward(self._make_ctx(self._upload(b.host), b, self._workspaces), b.rows_view)
+        if entry == "seen":
+            if len(self._graphs) > MAX_GRAPHS:
+                self._graphs = {k: v for k, v in self._graphs.items() if v == "seen"}
+            n = len(b.host)
+            entry = _Graph(static=torch.zeros(n, dtype=torch.int32, device=self.env.device),
+                           pinned=torch.zeros(n, dtype=torch.int32).pin_memory(), copied=torch.cuda.Event())
+            entry.pinned.numpy()[:] = b.host
+            entry.static.copy_(entry.pinned, non_blocking=True)
+            ctx = self._make_ctx(entry.static, b, {})
+            torch.cuda.current_stream().synchronize()
+            entry.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(entry.graph):
+                entry.logits = self.model.forward(ctx, b.rows_view)
+            self._graphs[key] = entry
+        else:
+            entry.copied.synchronize()  # the previous copy out of the pinned buffer is done
+            entry.pinned.numpy()[:] = b.host
+            entry.static.copy_(entry.pinned, non_blocking=True)
+        entry.copied.record()
+        entry.graph.replay()
+        return entry.logits
+
+
+GRAPH_BLOCK_BUCKET = 16  # block tables of graphed steps are padded to a multiple of this many pages
+MAX_GRAPHS = 48
+
+
+@dataclass
+class _Graph:
+    static: torch.Tensor
+    pinned: torch.Tensor
+    copied: "torch.cuda.Event"
+    graph: Optional["torch.cuda.CUDAGraph"] = None
+    logits: Optional[torch.Tensor] = None
+
+
+@dataclass
+class HostBatch:
+    host: np.ndarray
+    sizes: List[int]
+    offs: List[int]
+    n_tokens: int
+    n_seqs: int
+    n_rows: int
+    n_tiles: int
+    n_decode: int
+    max_blocks: int
+    max_kv: int
+    run_lengths: List[int]
+    first_positions: List[int]
+    slots: List[int]
+    rows_view: Optional[torch.Tensor] = None

@@ -23,6 +23,8 @@ from .spec import PartSpec
 
 @MIXERS.register("causal_self_attention")
 class CausalSelfAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
         p = spec.params

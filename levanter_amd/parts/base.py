@@ -124,6 +124,10 @@ class Mixer(Part):
     ``[T, dim]``) to the residual ``x`` (float32 ``[T, dim]``) in place; reads (and, if
     ``writes_cache``, first writes) ``unit``."""
 
+    graph_safe = False
+    """True if ``forward`` only launches work whose shape is fixed by the step's sizes and reads everything
+    else from device tensors (no host-side steering by ``ctx.host``): such steps may be captured into a HIP graph."""
+
     def cache_requirement(self):
         return None
 

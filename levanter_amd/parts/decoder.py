@@ -86,6 +86,10 @@ class DecoderLm:
                     raise ValueError(f"plan entry {i} reads cache unit {e.cache}, whose owner keeps something else ({a} vs {b})")
 
     @property
+    def graph_safe(self) -> bool:
+        return all(b.mixer.graph_safe for b in self.blocks)
+
+    @property
     def max_positions(self) -> Optional[int]:
         m = self.spec.max_positions
         e = self.embedding.max_positions

@@ -59,7 +59,15 @@ class Sampler:
         host[3 * r:] = np.asarray(positions, np.int64)
         t = torch.from_numpy(host)
         dev = t if self.device.type == "cpu" else t.pin_memory().to(self.device, non_blocking=True)
-        tokens = torch.empty(r, dtype=torch.int32, device=self.device)
-        logprobs = torch.empty(r, dtype=torch.float32, device=self.device)
+        out = torch.empty(2 * r, dtype=torch.int32, device=self.device)  # tokens, then log-probabilities: one copy back
+        tokens, logprobs = out[:r], out[r:].view(torch.float32)
         self.kernels.sample(logits, dev[:r].view(torch.float32), dev[r:3 * r].view(r, 2), dev[3 * r:], tokens, logprobs)
+        self._last_out = out
         return tokens, logprobs
+
+    def to_host(self, logits: torch.Tensor, temperatures, keys, positions) -> Tuple[list, list]:
+        """Sample and bring tokens and log-probabilities to the host with one copy (one synchronisation)."""
+        r = logits.shape[0]
+        self(logits, temperatures, keys, positions)
+        host = self._last_out.cpu()
+        return host[:r].tolist(), host[r:].view(torch.float32).tolist()

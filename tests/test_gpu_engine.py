@@ -410,3 +410,45 @@ def test_a_new_architecture_registers_without_touching_the_framework(tmp_path):
         assert len(res.tokens[0]) == 5
     finally:
         LmConfig.unregister("toy_gpt_rms")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_replayed_from_a_hip_graph_equal_eager_steps(dtype, monkeypatch):
+    """Steps of single tokens are captured into a HIP graph the second time their shape comes. Every replay
+    is compared with the same step run eagerly by a second runner, with eager work (a prompt portion of
+    another request, synchronisations) between the replays, and with pages that change from step to step."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import load_model, make_cache
+    import levanter_amd.engine.step as step_mod
+
+    monkeypatch.setattr(step_mod, "GRAPH_BLOCK_BUCKET", 4)  # so that the padded table width changes while decoding
+    d = write_model(TINY_B, 1, torch.float32 if dtype == "float32" else torch.bfloat16)
+    env = _env(dtype)
+    _, model = load_model(d, env)
+    cfg = InferenceEngineConfig(max_pages=40, max_seqs=4, page_size=16, max_pages_per_seq=16, compute_dtype=dtype)
+    runners = []
+    for graphs in (True, False):
+        cache = make_cache(model, cfg)
+        runners.append((ModelRunner(model, cache, env, use_graphs=graphs), cache))
+    assert runners[0][0].use_graphs and not runners[1][0].use_graphs
+    g = torch.Generator().manual_seed(9)
+    toks = {k: torch.randint(0, 1000, (120,), generator=g).tolist() for k in "abc"}
+    handles = [{k: c.open(k) for k in "abc"} for _, c in runners]
+    for (r, _), h in zip(runners, handles):
+        r.step([StepEntry(h["a"], toks["a"][:20], []), StepEntry(h["b"], toks["b"][:3], [])])
+    n_graph_steps = 0
+    for i in range(60):
+        outs = []
+        for (r, _), h in zip(runners, handles):
+            ia, ib = h["a"].length, h["b"].length
+            outs.append(r.step([StepEntry(h["a"], [toks["a"][ia]], [0]), StepEntry(h["b"], [toks["b"][ib]], [0])]).cpu())
+            if i % 7 == 3:  # eager work between the replays: a portion of a third request
+                ic = h["c"].length
+                r.step([StepEntry(h["c"], toks["c"][ic:ic + 5], [4])])
+                torch.cuda.synchronize()
+        torch.testing.assert_close(outs[0], outs[1], rtol=0, atol=0)
+        n_graph_steps += 1
+    graphs = [v for v in runners[0][0]._graphs.values() if v != "seen"]
+    assert len(graphs) >= 2  # the block-table bucket changed at least once while decoding 60 tokens
+    assert all(r.cache.groups[0].pool.n_free < 40 for r, _ in runners)
