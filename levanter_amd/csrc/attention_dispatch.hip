@@ -24,7 +24,7 @@ extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long 
   LEV_REQUIRE(H / KVH <= 16, "attention (matrix cores): at most 16 query heads per kv head, got %d", H / KVH);
   LEV_REQUIRE(HD % 16 == 0 && HD >= 16 && HD <= 128, "attention (matrix cores): head_dim=%d must be a multiple of 16 in 16..128", HD);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
-  LEV_REQUIRE(H <= 65535 && KVH <= 65535 && splits >= 1 && splits <= 65535, "attention: grid too large (heads=%d splits=%d)", H, splits);
+  LEV_REQUIRE(H <= 65535 && KVH <= 65535 && splits >= 1 && splits <= 64, "attention: grid too large (heads=%d) or more than 64 splits (%d)", H, splits);
   LEV_REQUIRE(window >= 0, "attention: window=%d must not be negative", window);
   LEV_REQUIRE(q_stride % 8 == 0 && o_stride % 4 == 0 && ((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
               "attention (matrix cores): q rows must be 16-byte aligned and out rows 8-byte aligned");

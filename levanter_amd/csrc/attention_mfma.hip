@@ -343,28 +343,36 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   }
 }
 
-// merge the splits of one (token, head) in the order of the splits
+// merge the splits of one (token, head): weights exp(m_z - max) per split, then a fixed-order sum
 __global__ void __launch_bounds__(64)
 LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __restrict__ decode_tokens,
                           const float* __restrict__ ws_m, const float* __restrict__ ws_l, const float* __restrict__ ws_o,
                           int H, int splits) {
-  const int idx = blockIdx.x, head = blockIdx.y;
+  __shared__ float wz[64];
+  const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const size_t slot0 = ((size_t)idx * H + head) * splits;
-  float mx = -INFINITY;
-  for (int z = 0; z < splits; ++z) mx = fmaxf(mx, ws_m[slot0 + z]);
-  float l = 0.f;
-  for (int z = 0; z < splits; ++z) {
-    const float mz = ws_m[slot0 + z];
-    if (mz != -INFINITY) l += ws_l[slot0 + z] * __expf(mz - mx);
-  }
+  const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
+  const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
+  const float mx = wave_max(mz);
+  const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
+  wz[lane] = w;
+  float l = lz * w;  // summed over the lanes in a fixed butterfly order
+  l = wave_sum(l);
+  __syncthreads();
   const float inv = 1.0f / l;
   bf16_t* orow = out + (size_t)decode_tokens[idx] * o_stride + (size_t)head * HD;
-  for (int d = threadIdx.x; d < HD; d += 64) {
+  for (int d = lane; d < HD; d += 64) {
     float acc = 0.f;
-    for (int z = 0; z < splits; ++z) {
-      const float mz = ws_m[slot0 + z];
-      if (mz != -INFINITY) acc += ws_o[(slot0 + z) * HD + d] * __expf(mz - mx);
+    int z = 0;
+    for (; z + 4 <= splits; z += 4) {
+      const float a0 = ws_o[(slot0 + z) * HD + d], a1 = ws_o[(slot0 + z + 1) * HD + d];
+      const float a2 = ws_o[(slot0 + z + 2) * HD + d], a3 = ws_o[(slot0 + z + 3) * HD + d];
+      acc += a0 * wz[z];
+      acc += a1 * wz[z + 1];
+      acc += a2 * wz[z + 2];
+      acc += a3 * wz[z + 3];
     }
+    for (; z < splits; ++z) acc += ws_o[(slot0 + z) * HD + d] * wz[z];
     orow[d] = float_to_bf16(acc * inv);
   }
 }

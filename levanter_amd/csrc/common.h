@@ -77,6 +77,14 @@ template <int NT> __device__ __forceinline__ float block_max(float v, float* red
   return t;
 }
 
+// A workgroup barrier that orders LDS traffic only. __syncthreads() also fences global memory, which makes
+// the compiler wait for every outstanding global load before the barrier and so defeats prefetching into
+// registers across it. Use this one between "LDS written" and "LDS read" phases when the global loads in
+// flight are private to the thread.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- activation functions, in 32-bit --------------------------------------------------------
 __device__ __forceinline__ float lev_activate(float u, int act) {
   switch (act) {

@@ -239,24 +239,31 @@ __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
   return a;
 }
 
+// Stage 1: block (row, part) scans its part of the vocabulary: best candidate, maximum of the scaled
+// logits and the sum of exp(scaled - that maximum). Stage 2: one wave per row merges the parts in order.
+#define SAMPLE_PARTS 64
+
 template <int NT>
-__global__ void sample_kernel(const float* __restrict__ logits, long row_stride, const float* __restrict__ temperature,
-                              const uint32_t* __restrict__ keys, const int* __restrict__ positions, int* __restrict__ tokens,
-                              float* __restrict__ logprobs, int V) {
+__global__ void __launch_bounds__(NT)
+sample_part_kernel(const float* __restrict__ logits, long row_stride, const float* __restrict__ temperature,
+                   const uint32_t* __restrict__ keys, const int* __restrict__ positions, float* __restrict__ part, int V) {
   __shared__ float red[NT / 64];
   __shared__ float sv[NT / 64];
   __shared__ int si[NT / 64];
-  const int r = blockIdx.x;
+  const int r = blockIdx.x, b = blockIdx.y;
   const float* lg = logits + (size_t)r * row_stride;
   const float temp = temperature[r];
   const bool greedy = (temp == 0.0f);
   const float safe_t = greedy ? 1.0f : temp;
   const uint32_t k0 = keys[2 * r], k1 = keys[2 * r + 1];
   const uint32_t pos = (uint32_t)positions[r];
+  const int groups = (V + 3) / 4;
+  const int per = (groups + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+  const int g_begin = b * per, g_end = min(groups, g_begin + per);
 
   ArgMax best = {-INFINITY, 0x7fffffff};
   float mx = -INFINITY;
-  for (int g = threadIdx.x; g * 4 < V; g += NT) {
+  for (int g = g_begin + threadIdx.x; g < g_end; g += NT) {
     uint32_t rnd[4] = {0, 0, 0, 0};
     if (!greedy) philox4x32_10((uint32_t)g, pos, 0u, 0u, k0, k1, rnd);
 #pragma unroll
@@ -270,7 +277,6 @@ __global__ void sample_kernel(const float* __restrict__ logits, long row_stride,
       }
     }
   }
-  // block argmax
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     ArgMax other = {__shfl_xor(best.v, o, 64), __shfl_xor(best.i, o, 64)};
@@ -285,20 +291,59 @@ __global__ void sample_kernel(const float* __restrict__ logits, long row_stride,
 #pragma unroll
   for (int i = 1; i < NT / 64; ++i) top = better(top, ArgMax{sv[i], si[i]});
   float se = 0.f;
-  for (int v = threadIdx.x; v < V; v += NT) se += expf(lg[v] / safe_t - mx);
+  if (mx != -INFINITY)
+    for (int g = g_begin + threadIdx.x; g < g_end; g += NT)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int v = g * 4 + j;
+        if (v < V) se += expf(lg[v] / safe_t - mx);
+      }
   se = block_sum<NT>(se, red);
   if (threadIdx.x == 0) {
-    const int tok = top.i < V ? top.i : 0;
-    tokens[r] = tok;
-    logprobs[r] = lg[tok] / safe_t - mx - logf(se);
+    float* p = part + ((size_t)r * SAMPLE_PARTS + b) * 4;
+    p[0] = top.v;
+    p[1] = __int_as_float(top.i);
+    p[2] = mx;
+    p[3] = se;
   }
 }
 
+__global__ void __launch_bounds__(64)
+sample_merge_kernel(const float* __restrict__ logits, long row_stride, const float* __restrict__ temperature,
+                    const float* __restrict__ part, int* __restrict__ tokens, float* __restrict__ logprobs, int V) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  const float* p = part + ((size_t)r * SAMPLE_PARTS + lane) * 4;
+  ArgMax best = {p[0], __float_as_int(p[1])};
+  const float mxb = p[2], seb = p[3];
+  const float mx = wave_max(mxb);
+  const float se = wave_sum(mxb == -INFINITY ? 0.f : seb * expf(mxb - mx));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ArgMax other = {__shfl_xor(best.v, o, 64), __shfl_xor(best.i, o, 64)};
+    best = better(best, other);
+  }
+  if (lane == 0) {
+    const float temp = temperature[r];
+    const float safe_t = temp == 0.0f ? 1.0f : temp;
+    const int tok = best.i < V ? best.i : 0;
+    tokens[r] = tok;
+    logprobs[r] = logits[(size_t)r * row_stride + tok] / safe_t - mx - logf(se);
+  }
+}
+
+extern "C" long lev_sample_workspace(int R) { return (long)R * SAMPLE_PARTS * 4 * (long)sizeof(float); }
+
 extern "C" int lev_sample(const float* logits, long row_stride, const float* temperature, const uint32_t* keys,
-                          const int* positions, int* tokens, float* logprobs, int R, int V, hipStream_t stream) {
+                          const int* positions, int* tokens, float* logprobs, float* workspace, int R, int V,
+                          hipStream_t stream) {
   LEV_REQUIRE(R >= 0 && V > 0, "sample: bad sizes rows=%d vocab=%d", R, V);
   LEV_REQUIRE(row_stride >= V, "sample: row stride %ld is smaller than the vocabulary %d", row_stride, V);
+  LEV_REQUIRE(R <= 65535 * 16, "sample: too many rows (%d)", R);
   if (R == 0) return 0;
-  sample_kernel<256><<<R, 256, 0, stream>>>(logits, row_stride, temperature, keys, positions, tokens, logprobs, V);
-  return lev_check_launch("sample");
+  LEV_REQUIRE(workspace != nullptr, "sample: a workspace of lev_sample_workspace(rows) bytes is needed");
+  static_assert(SAMPLE_PARTS == 64, "the merge kernel reads one part per lane");
+  sample_part_kernel<256><<<dim3(R, SAMPLE_PARTS), 256, 0, stream>>>(logits, row_stride, temperature, keys, positions, workspace, V);
+  if (int rc = lev_check_launch("sample")) return rc;
+  sample_merge_kernel<<<R, 64, 0, stream>>>(logits, row_stride, temperature, workspace, tokens, logprobs, V);
+  return lev_check_launch("sample merge");
 }

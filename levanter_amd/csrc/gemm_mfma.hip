@@ -32,111 +32,242 @@ __device__ __forceinline__ void epilogue_store(float v, int m, int n, const floa
 }
 
 // ------------------------------------------------------------------------------------------------
-#define TM 128
-#define TN 128
-#define TK 32
-#define LDS_STRIDE 40  // bf16 elements per LDS row: 32 + 8 of padding (80 bytes) against bank conflicts
+// Tile kernel. A workgroup of 4 waves (2 x 2) computes a BM x BN tile; a wave computes (BM/2) x (BN/2)
+// with 32x32x16 MFMA. The larger the wave's tile, the fewer LDS bytes per MFMA: 64 x 64 per wave needs
+// the whole LDS bandwidth, 128 x 128 half of it. Operand tiles of BK = 64 go global -> registers -> LDS
+// (two LDS buffers, one barrier per k-tile); the next tile's global loads are in flight during the products.
+// Workgroups are numbered so that each XCD (id % 8) works on a contiguous band of tiles and shares
+// operands in its own L2.
+#define TK 64
+#define LDS_STRIDE 72  // bf16 elements per LDS row: 64 + 8 of padding (144 bytes): 16-byte reads without bank conflicts
 
 template <typename TO>
+__device__ __forceinline__ void store_vec4(TO* p, const float v[4]);
+template <>
+__device__ __forceinline__ void store_vec4<float>(float* p, const float v[4]) {
+  *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void store_vec4<bf16_t>(bf16_t* p, const float v[4]) {
+  typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+  *reinterpret_cast<u32x2*>(p) = u32x2{(uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16),
+                                       (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16)};
+}
+
+template <typename TO, int BM, int BN>
 __global__ void __launch_bounds__(256)
 gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-                 const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][TM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][TN * LDS_STRIDE];
+                 const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act, int tiles_m, int tiles_n,
+                 int vec_ok) {
+  constexpr int WM = BM / 2, WN = BN / 2;    // the wave's tile
+  constexpr int TI = WM / 32, TJ = WN / 32;  // in 32 x 32 MFMA tiles
+  constexpr int CA = BM * (TK / 8) / 256;    // 16-byte chunks of the a tile per thread
+  constexpr int CW = BN * (TK / 8) / 256;
+  constexpr int CS = WN + 4;                 // row stride (floats) of a wave's output staging area
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+  bf16_t* As = smem;                               // [2][BM * LDS_STRIDE]
+  bf16_t* Ws = smem + 2 * BM * LDS_STRIDE;         // [2][BN * LDS_STRIDE]
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  // XCD-aware numbering: hardware sends consecutive workgroup ids to the 8 XCDs in turn
+  const int n_tiles = tiles_m * tiles_n;
+  int id = blockIdx.x;
+  if (n_tiles % 8 == 0) id = (id % 8) * (n_tiles / 8) + id / 8;
+  const int m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
 
-  // this thread's two 16-byte chunks of each operand tile
-  int lrow[2], lk[2];
+  // global -> registers: rows beyond the matrix and chunks beyond K read a valid address and become zero
+  uint32_t pa[CA], pw[CW];  // element offsets of this thread's rows (the launcher checks that they fit 32 bits)
+  bool oka[CA], okw[CW];
+  int kc[CA > CW ? CA : CW];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < CA; ++i) {
     const int c = tid + 256 * i;
-    lrow[i] = c >> 2;
-    lk[i] = (c & 3) * 8;
+    const int m = m0 + (c >> 3);
+    oka[i] = m < M;
+    pa[i] = (uint32_t)((size_t)(oka[i] ? m : M - 1) * lda);
+    kc[i] = (c & 7) * 8;
   }
-  u32x4 ra[2], rw[2];
-  auto gload = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int k = k0 + lk[i];
-      const int m = m0 + lrow[i], n = n0 + lrow[i];
-      ra[i] = (m < M && k < K) ? load16(a + (size_t)m * lda + k) : u32x4{0, 0, 0, 0};
-      rw[i] = (n < N && k < K) ? load16(w + (size_t)n * K + k) : u32x4{0, 0, 0, 0};
+  for (int i = 0; i < CW; ++i) {
+    const int c = tid + 256 * i;
+    const int n = n0 + (c >> 3);
+    okw[i] = n < N;
+    pw[i] = (uint32_t)((size_t)(okw[i] ? n : N - 1) * K);
+    kc[i] = (c & 7) * 8;
+  }
+  // Two register sets: while tile kt is multiplied out of LDS, the loads of tile kt + 2 are issued into one
+  // set and the other set (tile kt + 1, loaded one iteration ago) is written to the free LDS buffer between
+  // the products. A load has more than a whole iteration to arrive.
+  u32x4 ra[2][CA], rw[2][CW];
+  auto gload = [&](int set, int k0) {
+#pragma unroll
+    for (int i = 0; i < CA; ++i) {
+      const int k = k0 + kc[i];
+      ra[set][i] = load16(a + pa[i] + (k < K ? k : K - 8));  // masked when it is written to LDS: no wait for it here
+    }
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      const int k = k0 + kc[i];
+      rw[set][i] = load16(w + pw[i] + (k < K ? k : K - 8));
     }
   };
-  auto lstore = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      *reinterpret_cast<u32x4*>(&As[buf][lrow[i] * LDS_STRIDE + lk[i]]) = ra[i];
-      *reinterpret_cast<u32x4*>(&Ws[buf][lrow[i] * LDS_STRIDE + lk[i]]) = rw[i];
+  // chunk `i` of (CA + CW) of a register set goes to LDS buffer `buf`
+  auto lstore_one = [&](int set, int buf, int k0, int i) {
+    if (i < CA) {
+      const int c = tid + 256 * i;
+      const bool ok = oka[i] && k0 + kc[i] < K;
+      *reinterpret_cast<u32x4*>(&As[buf * BM * LDS_STRIDE + (c >> 3) * LDS_STRIDE + (c & 7) * 8]) = ok ? ra[set][i] : u32x4{0, 0, 0, 0};
+    } else {
+      const int j = i - CA;
+      const int c = tid + 256 * j;
+      const bool ok = okw[j] && k0 + kc[j] < K;
+      *reinterpret_cast<u32x4*>(&Ws[buf * BN * LDS_STRIDE + (c >> 3) * LDS_STRIDE + (c & 7) * 8]) = ok ? rw[set][j] : u32x4{0, 0, 0, 0};
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int nk = (K + TK - 1) / TK;
-  gload(0);
-  lstore(0);
-  __syncthreads();
+  gload(0, 0);
+#pragma unroll
+  for (int i = 0; i < CA + CW; ++i) lstore_one(0, 0, 0, i);
+  gload(1, min(1, nk - 1) * TK);
+  lds_barrier();
   const int fr = lane & 31, fk = (lane >> 5) * 8;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) gload((kt + 1) * TK);
-#pragma unroll
-    for (int ks = 0; ks < TK / 16; ++ks) {
-      bf16x8 af[2], wf[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        af[i] = as_bf16x8(*reinterpret_cast<const u32x4*>(&As[buf][(wm * 64 + i * 32 + fr) * LDS_STRIDE + ks * 16 + fk]));
-        wf[i] = as_bf16x8(*reinterpret_cast<const u32x4*>(&Ws[buf][(wn * 64 + i * 32 + fr) * LDS_STRIDE + ks * 16 + fk]));
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < nk) lstore(buf ^ 1);
-    __syncthreads();
-  }
+  constexpr int KS = TK / 16;
+  constexpr int PER = (CA + CW + KS - 1) / KS;  // LDS writes issued after each k-step's products
 
-  // 32x32 accumulator: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+  // one k-tile: `cur` is the register set that holds tile kt + 1, the other set receives tile kt + 2
+  auto ktile = [&](int kt, int cur) {
+    const int buf = kt & 1;
+    // always issued (past the end it re-reads the last tile, which is never stored): a conditional load would
+    // make the compiler's wait counters conservative at the join and serialise the two register sets
+    gload(cur ^ 1, min(kt + 2, nk - 1) * TK);
+    __builtin_amdgcn_sched_barrier(0);
+    const bf16_t* Ab = As + buf * BM * LDS_STRIDE + (wm * WM + fr) * LDS_STRIDE + fk;
+    const bf16_t* Wb = Ws + buf * BN * LDS_STRIDE + (wn * WN + fr) * LDS_STRIDE + fk;
+    // the fragments of k-step ks + 1 are read from LDS before the products of k-step ks are issued
+    u32x4 af[2][TI], wf[2][TJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TI; ++i) af[0][i] = *reinterpret_cast<const u32x4*>(Ab + i * 32 * LDS_STRIDE);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
-      if (n >= N) continue;
+    for (int j = 0; j < TJ; ++j) wf[0][j] = *reinterpret_cast<const u32x4*>(Wb + j * 32 * LDS_STRIDE);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (m < M) epilogue_store<TO>(acc[i][j][r], m, n, bias, residual, ldr, out, ldo, act);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = ks & 1, nx = c ^ 1;
+      if (ks + 1 < KS) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) af[nx][i] = *reinterpret_cast<const u32x4*>(Ab + i * 32 * LDS_STRIDE + (ks + 1) * 16);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) wf[nx][j] = *reinterpret_cast<const u32x4*>(Wb + j * 32 * LDS_STRIDE + (ks + 1) * 16);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads of the next k-step ahead of this k-step's products
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(af[c][i]), as_bf16x8(wf[c][j]), acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int q = 0; q < PER; ++q)  // after the last tile this writes the unused buffer
+        if (ks * PER + q < CA + CW) lstore_one(cur, buf ^ 1, (kt + 1) * TK, ks * PER + q);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    lds_barrier();  // not __syncthreads(): the loads of tile kt + 2 stay in flight across it
+  };
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    ktile(kt, 1);
+    ktile(kt + 1, 0);
+  }
+  if (kt < nk) ktile(kt, 1);
+
+  // Epilogue through LDS (the operand buffers are free now): each wave stages 32 rows of its tile at a time
+  // and writes them out as rows of 4 consecutive columns per lane, so that stores are wide and coalesced.
+  // 32x32 accumulator: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+  float* Cs = reinterpret_cast<float*>(smem) + wave * 32 * CS;
+#pragma unroll
+  for (int i = 0; i < TI; ++i) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Cs[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * CS + j * 32 + (lane & 31)] = acc[i][j][r];
+    __syncthreads();
+    for (int idx = lane; idx < 32 * (WN / 4); idx += 64) {
+      const int row = idx / (WN / 4), c4 = idx % (WN / 4);
+      const int m = m0 + wm * WM + i * 32 + row;
+      const int n = n0 + wn * WN + c4 * 4;
+      if (m >= M || n >= N) continue;
+      const f32x4 cv = *reinterpret_cast<const f32x4*>(&Cs[row * CS + c4 * 4]);
+      float v[4] = {cv[0], cv[1], cv[2], cv[3]};
+      if (vec_ok && n + 3 < N) {
+        if (bias) {
+          const f32x4 b = *reinterpret_cast<const f32x4*>(bias + n);
+          v[0] += b[0]; v[1] += b[1]; v[2] += b[2]; v[3] += b[3];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = lev_activate(v[e], act);
+        if (residual) {
+          const f32x4 rr = *reinterpret_cast<const f32x4*>(residual + (size_t)m * ldr + n);
+          v[0] += rr[0]; v[1] += rr[1]; v[2] += rr[2]; v[3] += rr[3];
+        }
+        store_vec4<TO>(out + (size_t)m * ldo + n, v);
+      } else {
+        for (int e = 0; e < 4 && n + e < N; ++e) epilogue_store<TO>(v[e], m, n + e, bias, residual, ldr, out, ldo, act);
       }
     }
+  }
+}
+
+template <typename TO, int BM, int BN>
+static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
+                       long ldo, int M, int N, int K, int act, hipStream_t stream) {
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const size_t lds_ops = (size_t)2 * (BM + BN) * LDS_STRIDE * sizeof(bf16_t);
+  const size_t lds_out = (size_t)4 * 32 * (BN / 2 + 4) * sizeof(float);
+  const size_t lds = lds_ops > lds_out ? lds_ops : lds_out;
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_tile_kernel<TO, BM, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return lev_fail("linear: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured = true;
+  }
+  // rows of 4 outputs are stored (and bias / residual read) as vectors when everything is aligned for it
+  const int vec_ok = (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) &&
+                     (!bias || ((uintptr_t)bias & 15) == 0);
+  gemm_tile_kernel<TO, BM, BN><<<tiles_m * tiles_n, 256, lds, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act,
+                                                                        tiles_m, tiles_n, vec_ok);
+  return 0;
 }
 
 // ------------------------------------------------------------------------------------------------
 // Skinny kernel. WAVES waves per workgroup; wave v takes the 32-wide k-steps v, v + WAVES, ...
-// MT = number of 16-row tiles of `a` (1..4).
-template <typename TO, int WAVES, int MT>
+// MT = number of 16-row tiles of `a` (1..4); NT = number of 16-column tiles per workgroup (each wave
+// computes all of them from one load of its `a` fragments); U = k-steps whose loads are in flight together.
+template <typename TO, int WAVES, int MT, int NT, int U>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
-  __shared__ f32x4 red[WAVES][MT][64];
+  __shared__ f32x4 red[WAVES][NT][MT][64];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int fr = lane & 15, fk = (lane >> 4) * 8;
-  const int n = n0 + fr;
-  const bool n_ok = n < N;
-  const bf16_t* wrow = w + (size_t)(n_ok ? n : 0) * K;
+  const bf16_t* wrow[NT];
+  bool n_ok[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + j * 16 + fr;
+    n_ok[j] = n < N;
+    wrow[j] = w + (size_t)(n_ok[j] ? n : 0) * K;
+  }
   const bf16_t* arow[MT];
   bool m_ok[MT];
 #pragma unroll
@@ -145,42 +276,48 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
     m_ok[t] = m < M;
     arow[t] = a + (size_t)(m_ok[t] ? m : 0) * lda;
   }
-  f32x4 acc[MT];
+  f32x4 acc[NT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int nsteps = (K + 31) / 32;
-  constexpr int U = MT == 1 ? 8 : 4;  // k-steps whose loads are issued together (bytes in flight per wave)
   for (int s0 = wave; s0 < nsteps; s0 += WAVES * U) {
-    u32x4 wv[U];
+    u32x4 wv[U][NT];
     u32x4 av[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (s0 + u * WAVES) * 32 + fk;
       const bool k_ok = k < K;
-      wv[u] = (k_ok && n_ok) ? load16(wrow + k) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < NT; ++j) wv[u][j] = (k_ok && n_ok[j]) ? load16(wrow[j] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
       for (int t = 0; t < MT; ++t) av[u][t] = (k_ok && m_ok[t]) ? load16(arow[t] + k) : u32x4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av[u][t]), as_bf16x8(wv[u]), acc[t], 0, 0, 0);
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av[u][t]), as_bf16x8(wv[u][j]), acc[j][t], 0, 0, 0);
   }
 #pragma unroll
-  for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) red[wave][j][t][lane] = acc[j][t];
   __syncthreads();
-  // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16
-  for (int idx = tid; idx < MT * 64; idx += WAVES * 64) {
-    const int t = idx >> 6, l = idx & 63;
-    f32x4 s = red[0][t][l];
+  // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16. Partial sums are added in wave order.
+  for (int idx = tid; idx < NT * MT * 64; idx += WAVES * 64) {
+    const int l = idx & 63, t = (idx >> 6) % MT, j = (idx >> 6) / MT;
+    f32x4 s = red[0][j][t][l];
 #pragma unroll
     for (int v = 1; v < WAVES; ++v) {
-      const f32x4 o = red[v][t][l];
+      const f32x4 o = red[v][j][t][l];
       s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
     }
-    const int nn = n0 + (l & 15);
+    const int nn = n0 + j * 16 + (l & 15);
     if (nn >= N) continue;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -190,18 +327,24 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   }
 }
 
-template <typename TO, int WAVES>
+// Choices measured on MI355X at K = 4096 .. 16384 (weights streamed at 4 - 6 TB/s for M <= 16):
+//   M <= 16: one column tile per workgroup, 8 loads in flight per wave;
+//   M  > 32: the `a` fragments cost more than the weights, so two column tiles share them when N is
+//            large enough to still fill the chip, and 16 waves split K when N is small.
+template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
-  const int grid = (N + 15) / 16;
   const int mt = (M + 15) / 16;
-#define LEV_SKINNY(MT_) \
-  gemm_skinny_kernel<TO, WAVES, MT_><<<grid, WAVES * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act)
-  switch (mt) {
-    case 1: LEV_SKINNY(1); break;
-    case 2: LEV_SKINNY(2); break;
-    case 3: LEV_SKINNY(3); break;
-    default: LEV_SKINNY(4); break;
+  const int tiles = (N + 15) / 16;
+#define LEV_SKINNY(WAVES_, MT_, NT_, U_)                                                                            gemm_skinny_kernel<TO, WAVES_, MT_, NT_, U_><<<(tiles + NT_ - 1) / NT_, WAVES_ * 64, 0, stream>>>(a, lda, w, bias, residual,                                                                                                    ldr, out, ldo, M, N, K, act)
+  if (mt == 1) {
+    if (tiles >= 1024) LEV_SKINNY(4, 1, 1, 8); else LEV_SKINNY(8, 1, 1, 8);
+  } else if (mt == 2) {
+    if (tiles >= 1024) LEV_SKINNY(4, 2, 1, 4); else LEV_SKINNY(8, 2, 1, 4);
+  } else if (tiles >= 512) {
+    if (mt == 3) LEV_SKINNY(8, 3, 2, 2); else LEV_SKINNY(8, 4, 2, 2);
+  } else {
+    if (mt == 3) LEV_SKINNY(16, 3, 1, 2); else LEV_SKINNY(16, 4, 1, 2);
   }
 #undef LEV_SKINNY
 }
@@ -210,14 +353,21 @@ template <typename TO>
 static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                              TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
   if (M <= 64) {
-    if ((N + 15) / 16 >= 1024)
-      launch_skinny<TO, 4>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
-    else
-      launch_skinny<TO, 8>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    launch_skinny<TO>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
   } else {
-    dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
-    if (grid.y > 65535) return lev_fail("linear: too many rows (%d) for one launch", M);
-    gemm_tile_kernel<TO><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
+    if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
+      return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
+    // the largest tile that still gives every CU (256 of them) a workgroup
+    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const long t128 = (long)((M + 255) / 256) * ((N + 127) / 128);
+    int rc;
+    if (M > 128 && t256 >= 256)
+      rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    else if (M > 128 && t128 >= 192)
+      rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    else
+      rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    if (rc) return rc;
   }
   return lev_check_launch("linear_mfma");
 }

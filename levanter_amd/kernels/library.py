@@ -67,7 +67,8 @@ class HipKernels:
             "lev_embed": [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p],
             "lev_norm": [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_int, c_void_p],
             "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
-            "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+            "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+            "lev_sample_workspace": [c_int],
             "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
             "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
             + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
@@ -79,8 +80,9 @@ class HipKernels:
         for name, args in sigs.items():
             fn = getattr(L, name)
             fn.argtypes = args
-            fn.restype = c_long if name == "lev_attention_mfma_workspace" else c_int
+            fn.restype = c_long if name.endswith("_workspace") else c_int
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
+        self._sample_ws = None
 
     def _check(self, rc: int) -> None:
         if rc != 0:
@@ -209,8 +211,12 @@ class HipKernels:
         _req(positions.dtype == torch.int32 and positions.numel() == R, "sample: one int32 position per row")
         _req(out_tokens.dtype == torch.int32 and out_tokens.numel() == R, "sample: tokens out must be int32 [R]")
         _req(out_logprobs.dtype == torch.float32 and out_logprobs.numel() == R, "sample: logprobs out must be float32 [R]")
+        need = self.lib.lev_sample_workspace(R)
+        if self._sample_ws is None or self._sample_ws.numel() < need or self._sample_ws.device != logits.device:
+            self._sample_ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=logits.device)
         self._check(self.lib.lev_sample(_ptr(logits), _rows(logits, "sample: logits"), _ptr(temperatures), _ptr(keys),
-                                        _ptr(positions), _ptr(out_tokens), _ptr(out_logprobs), R, V, _stream()))
+                                        _ptr(positions), _ptr(out_tokens), _ptr(out_logprobs), _ptr(self._sample_ws), R, V,
+                                        _stream()))
 
 
 _KERNELS = None
