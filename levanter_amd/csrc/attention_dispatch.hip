@@ -2,24 +2,28 @@
 #include "common.h"
 
 #define LEV_DECL(HDV)                                                                                                       \
-  extern "C" int lev_attention_mfma_hd##HDV(const void*, long, void*, long, const void*, const void*, const int*, const int*, \
-                                            const int*, int, const int*, int, const int*, int, void*, int, int, int, int,    \
-                                            float, int, hipStream_t);
+  extern "C" int lev_attention_mfma_hd##HDV(const void*, long, void*, long, void*, void*, const int*, const int*, const int*, \
+                                            int, const int*, int, const int*, int, const void*, const void*, long, const int*, \
+                                            void*, int, int, int, int, float, int, hipStream_t);
 LEV_DECL(16) LEV_DECL(32) LEV_DECL(48) LEV_DECL(64) LEV_DECL(80) LEV_DECL(96) LEV_DECL(112) LEV_DECL(128)
 #undef LEV_DECL
 
-// bytes of workspace for `rows` = decode tokens x splits partial results of H heads
-extern "C" long lev_attention_mfma_workspace(int rows, int H, int HD) {
-  return (long)rows * H * (HD + 2) * (long)sizeof(float);
+// bytes of workspace for n_decode single-token queries in `splits` splits: the counters of the (token, kv head)
+// pairs, which must be zero before the first launch (every launch leaves them zero), then the partial results
+// (the counters have a fixed place and size so that launches of different shapes can share one workspace)
+#define LEV_ATTN_COUNTERS 65536
+extern "C" long lev_attention_mfma_workspace(int n_decode, int splits, int H, int KVH, int HD) {
+  return ((long)LEV_ATTN_COUNTERS + (long)n_decode * splits * H * (HD + 2)) * (long)sizeof(float);
 }
+extern "C" int lev_attention_mfma_max_split_rows() { return LEV_ATTN_COUNTERS; }
 
 extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
 
-extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long o_stride, const void* k_pages,
-                                  const void* v_pages, const int* positions, const int* token_seq, const int* block_tables,
-                                  int bt_stride, const int* prefill_tiles, int n_prefill_tiles, const int* decode_tokens,
-                                  int n_decode, void* workspace, int H, int KVH, int HD, int PS, int splits, float scale,
-                                  int window, hipStream_t stream) {
+extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long o_stride, void* k_pages, void* v_pages,
+                                  const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
+                                  const int* prefill_tiles, int n_prefill_tiles, const int* decode_tokens, int n_decode,
+                                  const void* k_new, const void* v_new, long kv_stride, const int* dest, void* workspace, int H,
+                                  int KVH, int HD, int PS, int splits, float scale, int window, hipStream_t stream) {
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(H / KVH <= 16, "attention (matrix cores): at most 16 query heads per kv head, got %d", H / KVH);
   LEV_REQUIRE(HD % 16 == 0 && HD >= 16 && HD <= 128, "attention (matrix cores): head_dim=%d must be a multiple of 16 in 16..128", HD);
@@ -31,11 +35,17 @@ extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long 
   LEV_REQUIRE(n_prefill_tiles == 0 || prefill_tiles, "attention: prefill tiles are missing");
   LEV_REQUIRE(n_decode == 0 || decode_tokens, "attention: decode tokens are missing");
   LEV_REQUIRE(n_decode == 0 || splits == 1 || workspace, "attention: split decoding needs a workspace");
+  LEV_REQUIRE(splits == 1 || (long)n_decode * KVH <= LEV_ATTN_COUNTERS,
+              "attention: split decoding of %d tokens x %d kv heads exceeds the %d counters of the workspace", n_decode, KVH,
+              LEV_ATTN_COUNTERS);
+  LEV_REQUIRE((k_new == nullptr) == (v_new == nullptr), "attention: new keys and values come together");
+  LEV_REQUIRE(!k_new || (n_prefill_tiles == 0 && dest && kv_stride % 8 == 0 && ((uintptr_t)k_new & 15) == 0),
+              "attention: new keys and values in the same launch need a step of single tokens, destinations and 16-byte aligned rows");
 #define LEV_CASE(HDV)                                                                                                     \
   case HDV:                                                                                                               \
     return lev_attention_mfma_hd##HDV(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables,    \
-                                      bt_stride, prefill_tiles, n_prefill_tiles, decode_tokens, n_decode, workspace, H, KVH, \
-                                      PS, splits, scale, window, stream);
+                                      bt_stride, prefill_tiles, n_prefill_tiles, decode_tokens, n_decode, k_new, v_new,      \
+                                      kv_stride, dest, workspace, H, KVH, PS, splits, scale, window, stream);
   switch (HD) {
     LEV_CASE(16) LEV_CASE(32) LEV_CASE(48) LEV_CASE(64) LEV_CASE(80) LEV_CASE(96) LEV_CASE(112) LEV_CASE(128)
   }

@@ -235,15 +235,23 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
 
 // ------------------------------------------------------------------------------------------------
 // Decode: one wave per (token, kv head, split). Columns of Q^T are the G = H / KVH query heads that
-// share the kv head. Partial results go to the workspace when there is more than one split:
-//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD]
+// share the kv head. With more than one split the partial results go to the workspace
+//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD], counters [token][kv head]
+// and the wave that finishes last (an atomic ticket; nobody waits) merges them in the order of the
+// splits: the result does not depend on which wave that is. It resets the counter for the next launch.
+//
+// k_new != null: the step's new key and value of each token are not in the cache yet. The wave whose key
+// range holds the token's own position takes them from k_new / v_new (rows of the projection's output),
+// uses them in place of what the cache holds there, and writes them to dest[t] = page * PS + offset.
 __global__ void __launch_bounds__(64)
 LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
-                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-                         const int* __restrict__ positions, const int* __restrict__ token_seq,
-                         const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ decode_tokens,
-                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o, int H, int KVH, int PS,
-                         int splits, float scale, int window) {
+                         bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
+                         const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
+                         const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
+                         const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
+                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o, int* __restrict__ counters,
+                         int H, int KVH, int PS, int splits, float scale, int window) {
+  __shared__ float wz[64];
   const int lane = threadIdx.x;
   const int fr = lane & 15, g = lane >> 4;
   const int idx = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
@@ -257,6 +265,23 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   const int kb_begin = kb_first + z * per, kb_end = min(kb_last + 1, kb_begin + per);
   const int head = kvh * G + fr;  // this lane's query head (column of Q^T)
   const int q_pos = fr < G ? pos : -1;
+  const size_t head_elems = (size_t)HD * PS;
+  const bool fused = k_new != nullptr;
+  const bool owner = fused && kb_begin <= kb_last && kb_last < kb_end;  // this wave's range holds the token's position
+  const bf16_t* kn = fused ? k_new + (size_t)t * kv_stride + (size_t)kvh * HD : nullptr;
+  const bf16_t* vn = fused ? v_new + (size_t)t * kv_stride + (size_t)kvh * HD : nullptr;
+
+  if (owner) {  // the new key and value go to their page (read by later steps only)
+    const int dst = dest[t];
+    if (dst >= 0) {
+      bf16_t* kb_ = k_pages + ((size_t)(dst / PS) * KVH + kvh) * head_elems;
+      bf16_t* vb_ = v_pages + ((size_t)(dst / PS) * KVH + kvh) * head_elems;
+      const int off = dst % PS;
+      for (int c = lane; c < NCHUNK; c += 64)
+        *reinterpret_cast<u32x4*>(kb_ + ((size_t)c * PS + off) * 8) = *reinterpret_cast<const u32x4*>(kn + c * 8);
+      for (int d = lane; d < HD; d += 64) vb_[(size_t)d * PS + off] = vn[d];
+    }
+  }
 
   u32x4 qf[NKS];
 #pragma unroll
@@ -269,7 +294,6 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
 #pragma unroll
   for (int i = 0; i < NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const size_t head_elems = (size_t)HD * PS;
 
   for (int kb = kb_begin; kb < kb_end; ++kb) {
     const int key0 = kb * 64;
@@ -281,12 +305,14 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
       for (int hh = 0; hh < 2; ++hh) {
         const int kp = key0 + tile_key(u, hh, fr);
         const bool ok = kp <= pos && kp >= lo;
+        const bool is_new = fused && kp == pos;
         const int page = ok ? bt[kp / PS] : -1;
-        const bf16_t* base = k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp % PS) * 8;
+        const bf16_t* base = is_new ? kn : k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp % PS) * 8;
+        const size_t cstride = is_new ? 8 : (size_t)PS * 8;
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
           const int c = 4 * s + g;
-          kf[u][hh][s] = (page >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(base + (size_t)c * PS * 8) : u32x4{0, 0, 0, 0};
+          kf[u][hh][s] = (page >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(base + (size_t)c * cstride) : u32x4{0, 0, 0, 0};
         }
       }
     // value operands: tile dt, row fr is head dim 16*dt + fr, k-slots are keys 32u + 8g .. +7
@@ -297,9 +323,23 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
       const bool ok = kp <= pos && kp + 7 >= lo;
       const int page = ok ? bt[kp / PS] : -1;
       const bf16_t* base = v_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + kp % PS;
+      const int jn = pos - kp;  // slot of the new value among this lane's 8 keys, if 0 <= jn < 8
+      const bool has_new = fused && jn >= 0 && jn < 8;
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-        vf[dt][u] = page >= 0 ? *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS) : u32x4{0, 0, 0, 0};
+      for (int dt = 0; dt < NDT; ++dt) {
+        u32x4 v = page >= 0 ? *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS) : u32x4{0, 0, 0, 0};
+        if (has_new) {
+          const uint32_t nv = vn[16 * dt + fr];
+          const int w = jn >> 1;
+          const uint32_t old = w == 0 ? v[0] : (w == 1 ? v[1] : (w == 2 ? v[2] : v[3]));
+          const uint32_t neu = (jn & 1) ? ((old & 0x0000ffffu) | (nv << 16)) : ((old & 0xffff0000u) | nv);
+          v[0] = w == 0 ? neu : v[0];
+          v[1] = w == 1 ? neu : v[1];
+          v[2] = w == 2 ? neu : v[2];
+          v[3] = w == 3 ? neu : v[3];
+        }
+        vf[dt][u] = v;
+      }
     }
     f32x4 st[2][2];
 #pragma unroll
@@ -322,16 +362,19 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
-  if (q_pos < 0) return;
   if (splits == 1) {
-    const float inv = 1.0f / l;
-    bf16_t* orow = out + (size_t)t * o_stride + (size_t)head * HD;
+    if (q_pos >= 0) {
+      const float inv = 1.0f / l;
+      bf16_t* orow = out + (size_t)t * o_stride + (size_t)head * HD;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      const u32x2 v = u32x2{pack_bf16(o[dt][0] * inv, o[dt][1] * inv), pack_bf16(o[dt][2] * inv, o[dt][3] * inv)};
-      *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * g) = v;
+      for (int dt = 0; dt < NDT; ++dt) {
+        const u32x2 v = u32x2{pack_bf16(o[dt][0] * inv, o[dt][1] * inv), pack_bf16(o[dt][2] * inv, o[dt][3] * inv)};
+        *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * g) = v;
+      }
     }
-  } else {
+    return;
+  }
+  if (q_pos >= 0) {
     const size_t slot = ((size_t)idx * H + head) * splits + z;
     if (g == 0) {
       ws_m[slot] = m;
@@ -341,48 +384,50 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(wo + 16 * dt + 4 * g) = o[dt];
   }
-}
-
-// merge the splits of one (token, head): weights exp(m_z - max) per split, then a fixed-order sum
-__global__ void __launch_bounds__(64)
-LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __restrict__ decode_tokens,
-                          const float* __restrict__ ws_m, const float* __restrict__ ws_l, const float* __restrict__ ws_o,
-                          int H, int splits) {
-  __shared__ float wz[64];
-  const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const size_t slot0 = ((size_t)idx * H + head) * splits;
-  const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
-  const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
-  const float mx = wave_max(mz);
-  const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
-  wz[lane] = w;
-  float l = lz * w;  // summed over the lanes in a fixed butterfly order
-  l = wave_sum(l);
-  __syncthreads();
-  const float inv = 1.0f / l;
-  bf16_t* orow = out + (size_t)decode_tokens[idx] * o_stride + (size_t)head * HD;
-  for (int d = lane; d < HD; d += 64) {
-    float acc = 0.f;
-    int z = 0;
-    for (; z + 4 <= splits; z += 4) {
-      const float a0 = ws_o[(slot0 + z) * HD + d], a1 = ws_o[(slot0 + z + 1) * HD + d];
-      const float a2 = ws_o[(slot0 + z + 2) * HD + d], a3 = ws_o[(slot0 + z + 3) * HD + d];
-      acc += a0 * wz[z];
-      acc += a1 * wz[z + 1];
-      acc += a2 * wz[z + 2];
-      acc += a3 * wz[z + 3];
+  // the last wave of this (token, kv head) to get here merges the splits
+  __threadfence();  // this wave's partial results are visible to the device before its ticket is
+  int ticket = 0;
+  if (lane == 0) ticket = __hip_atomic_fetch_add(&counters[idx * KVH + kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  ticket = __shfl(ticket, 0, 64);
+  if (ticket != splits - 1) return;
+  __threadfence();  // and the others' partial results are visible to this wave
+  if (lane == 0) counters[idx * KVH + kvh] = 0;
+  for (int hq = 0; hq < G; ++hq) {
+    const int hd_ = kvh * G + hq;
+    const size_t slot0 = ((size_t)idx * H + hd_) * splits;
+    const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
+    const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
+    const float mx = wave_max(mz);
+    const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
+    __syncthreads();  // one wave: orders the reuse of wz between heads
+    wz[lane] = w;
+    const float lsum = wave_sum(lz * w);
+    __syncthreads();
+    const float inv = 1.0f / lsum;
+    bf16_t* orow = out + (size_t)t * o_stride + (size_t)hd_ * HD;
+    for (int d = lane; d < HD; d += 64) {
+      float acc = 0.f;
+      int zz = 0;
+      for (; zz + 4 <= splits; zz += 4) {
+        const float a0 = ws_o[(slot0 + zz) * HD + d], a1 = ws_o[(slot0 + zz + 1) * HD + d];
+        const float a2 = ws_o[(slot0 + zz + 2) * HD + d], a3 = ws_o[(slot0 + zz + 3) * HD + d];
+        acc += a0 * wz[zz];
+        acc += a1 * wz[zz + 1];
+        acc += a2 * wz[zz + 2];
+        acc += a3 * wz[zz + 3];
+      }
+      for (; zz < splits; ++zz) acc += ws_o[(slot0 + zz) * HD + d] * wz[zz];
+      orow[d] = float_to_bf16(acc * inv);
     }
-    for (; z < splits; ++z) acc += ws_o[(slot0 + z) * HD + d] * wz[z];
-    orow[d] = float_to_bf16(acc * inv);
   }
 }
 
-extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, void* out, long o_stride, const void* k_pages,
-                                               const void* v_pages, const int* positions, const int* token_seq,
+extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, void* out, long o_stride, void* k_pages,
+                                               void* v_pages, const int* positions, const int* token_seq,
                                                const int* block_tables, int bt_stride, const int* prefill_tiles,
-                                               int n_prefill_tiles, const int* decode_tokens, int n_decode, void* workspace,
-                                               int H, int KVH, int PS, int splits, float scale, int window,
-                                               hipStream_t stream) {
+                                               int n_prefill_tiles, const int* decode_tokens, int n_decode, const void* k_new,
+                                               const void* v_new, long kv_stride, const int* dest, void* workspace, int H,
+                                               int KVH, int PS, int splits, float scale, int window, hipStream_t stream) {
   if (n_prefill_tiles > 0) {
     dim3 grid(n_prefill_tiles, H);
     LEV_NAME(attn_prefill_hd)<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
@@ -391,20 +436,18 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     if (int rc = lev_check_launch("attention prefill")) return rc;
   }
   if (n_decode > 0) {
+    // workspace: 65536 counters (zero between launches), then m, l, o of every (token, head, split)
     const size_t rows = (size_t)n_decode * H * splits;
-    float* ws_m = (float*)workspace;
+    int* counters = (int*)workspace;
+    float* ws_m = (float*)workspace + 65536;
     float* ws_l = ws_m + rows;
     float* ws_o = ws_l + rows;
     dim3 grid(n_decode, KVH, splits);
-    LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (const bf16_t*)k_pages,
-                                                      (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-                                                      decode_tokens, ws_m, ws_l, ws_o, H, KVH, PS, splits, scale, window);
+    LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages,
+                                                      (bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
+                                                      decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest,
+                                                      ws_m, ws_l, ws_o, counters, H, KVH, PS, splits, scale, window);
     if (int rc = lev_check_launch("attention decode")) return rc;
-    if (splits > 1) {
-      dim3 cgrid(n_decode, H);
-      LEV_NAME(attn_combine_hd)<<<cgrid, 64, 0, stream>>>((bf16_t*)out, o_stride, decode_tokens, ws_m, ws_l, ws_o, H, splits);
-      if (int rc = lev_check_launch("attention combine")) return rc;
-    }
   }
   return 0;
 }

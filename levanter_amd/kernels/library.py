@@ -74,8 +74,9 @@ class HipKernels:
             + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
             "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 5 + [c_void_p],
             "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                   c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 5 + [c_float, c_int, c_void_p],
-            "lev_attention_mfma_workspace": [c_int, c_int, c_int],
+                                   c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p]
+            + [c_int] * 5 + [c_float, c_int, c_void_p],
+            "lev_attention_mfma_workspace": [c_int] * 5,
         }
         for name, args in sigs.items():
             fn = getattr(L, name)
@@ -160,10 +161,15 @@ class HipKernels:
 
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,
-                        page_size: int, scale: float, window: Optional[int], block_tables) -> None:
+                        page_size: int, scale: float, window: Optional[int], block_tables, k_new=None, v_new=None,
+                        dest=None) -> bool:
         """Causal attention of the step's query tokens over the pages. ``meta`` is the step's
-        ``AttentionMeta`` (positions, token_seq and the work lists), block_tables int32 [S, B]."""
-        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq)
+        ``AttentionMeta`` (positions, token_seq and the work lists), block_tables int32 [S, B].
+
+        ``k_new``/``v_new``/``dest``: the step's new keys and values, not yet written. Returns True if this
+        call has written them to their pages (a step of single tokens on the matrix-core path does it inside
+        the attention kernel); False means the caller must call ``kv_write`` first and call again without them."""
+        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, k_new, v_new, dest)
         T = q.shape[0]
         _req(q.shape[1] == n_heads * head_dim and out.shape == q.shape, "attention: q and out must be [T, heads*head_dim]")
         _req(q.dtype == out.dtype == k_pages.dtype == v_pages.dtype and q.dtype in _DT, "attention: dtypes differ")
@@ -172,25 +178,39 @@ class HipKernels:
         _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
         w = int(window) if window else 0
         qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
-        if q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads):
+        mfma = q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
+        if k_new is not None:
+            fusable = mfma and meta.n_prefill_tiles == 0 and meta.n_decode == T
+            if not fusable:
+                return False
+            _req(k_new.shape == v_new.shape == (T, n_kv_heads * head_dim) and k_new.dtype == v_new.dtype == q.dtype,
+                 "attention: new keys and values must be [T, kv_heads*head_dim] of the compute dtype")
+            _req(dest is not None and dest.dtype == torch.int32 and dest.numel() == T, "attention: one int32 destination per token")
+            kvs = _rows(k_new, "attention: k_new")
+            _req(kvs == _rows(v_new, "attention: v_new"), "attention: new keys and values must share a row stride")
+        if mfma:
             splits = self.decode_splits(meta, n_heads, n_kv_heads)
-            need = self.lib.lev_attention_mfma_workspace(meta.n_decode * splits, n_heads, head_dim)
-            ws = meta.workspace(need, q.device)
+            need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
+            ws = meta.zeroed_workspace(need, q.device)
             self._check(self.lib.lev_attention_mfma(
                 _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles,
-                _ptr(meta.decode_tokens), meta.n_decode, _ptr(ws), n_heads, n_kv_heads, head_dim, page_size,
+                _ptr(meta.decode_tokens), meta.n_decode, _ptr(k_new), _ptr(v_new), kvs if k_new is not None else 0,
+                _ptr(dest) if k_new is not None else None, _ptr(ws), n_heads, n_kv_heads, head_dim, page_size,
                 splits, float(scale), w, _stream()))
-        else:
-            self._check(self.lib.lev_attention_simple(
-                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
-                _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, page_size, float(scale), w,
-                _DT[q.dtype], _stream()))
+            return k_new is not None
+        self._check(self.lib.lev_attention_simple(
+            _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
+            _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, page_size, float(scale), w,
+            _DT[q.dtype], _stream()))
+        return False
 
     @staticmethod
     def decode_splits(meta, n_heads: int, n_kv_heads: int) -> int:
         """Into how many key ranges a single-token query is split so that the chip is filled."""
         if meta.n_decode == 0:
+            return 1
+        if meta.n_decode * n_kv_heads > 65536:  # more (token, kv head) pairs than the workspace has counters: the chip is full anyway
             return 1
         want = max(1, 2048 // max(1, meta.n_decode * n_kv_heads))
         most = max(1, (meta.max_kv_len + 63) // 64)  # at least 64 keys per split

@@ -61,10 +61,15 @@ class CausalSelfAttention(Mixer):
         if self.rotary is not None:
             self.rotary.rotate(q, k, ctx)
         g = unit.group
-        if writes_cache:
-            ctx.kernels.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size)
         a = ctx.empty(h.shape[0], self.q_cols)
-        ctx.kernels.paged_attention(q, a, unit.k_pages, unit.v_pages, ctx.attention, n_heads=self.n_heads,
-                                    n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, page_size=g.page_size,
-                                    scale=self.scale, window=self.window, block_tables=g.block_tables)
+        args = dict(n_heads=self.n_heads, n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, page_size=g.page_size,
+                    scale=self.scale, window=self.window, block_tables=g.block_tables)
+        written = False
+        if writes_cache:  # a step of single tokens writes the new keys and values inside the attention kernel
+            written = ctx.kernels.paged_attention(q, a, unit.k_pages, unit.v_pages, ctx.attention, k_new=k, v_new=v,
+                                                  dest=g.dest, **args)
+        if not written:
+            if writes_cache:
+                ctx.kernels.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size)
+            ctx.kernels.paged_attention(q, a, unit.k_pages, unit.v_pages, ctx.attention, **args)
         self.out(a, ctx, residual=x)

@@ -123,7 +123,9 @@ class EmulatedKernels:
 
     # ---- attention
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads, n_kv_heads, head_dim, page_size, scale, window,
-                        block_tables, round_probs=None) -> None:
+                        block_tables, k_new=None, v_new=None, dest=None) -> bool:
+        if k_new is not None:
+            return False  # this stand-in never writes the cache inside attention: the caller calls kv_write
         T = q.shape[0]
         g = n_heads // n_kv_heads
         for t in range(T):
@@ -140,6 +142,7 @@ class EmulatedKernels:
                 p = p.to(torch.bfloat16).float()
             o = torch.einsum("hn,hnd->hd", p, vs)
             out[t] = o.reshape(-1).to(out.dtype)
+        return False
 
     # ---- sampling
     def sample(self, logits, temperatures, keys, positions, out_tokens, out_logprobs) -> None:

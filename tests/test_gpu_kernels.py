@@ -273,3 +273,51 @@ def test_sample_ties_and_frequencies(K):
     # the noise is the documented function of (key, position, entry)
     noise = gumbel_noise(3, 12345, 0, 5)
     assert int(toks[3]) == int(torch.argmax(base / t + noise))
+
+
+@pytest.mark.parametrize("H,KVH,HD,PS,kv_lens,window", [
+    (4, 4, 64, 16, [1, 17, 64, 65, 300], None),
+    (8, 2, 128, 16, [16, 33, 640], None),
+    (3, 3, 32, 32, [5, 100, 31, 32, 33], 40),
+])
+def test_decode_attention_that_writes_its_own_keys_and_values(K, H, KVH, HD, PS, kv_lens, window):
+    """A step of single tokens may hand the new keys and values to the attention kernel instead of writing
+    them first. Output and pages equal the two-kernel way; launches of different shapes share the workspace."""
+    dtype = torch.bfloat16
+    n_pages = sum((k + PS - 1) // PS for k in kv_lens) + 2
+    bt, kp, vp, kd, vd, ks, vs = _fill_cache(K, dtype, [k - 1 for k in kv_lens] if min(kv_lens) > 1 else kv_lens, KVH, HD, PS, n_pages, seed=3)
+    # caches hold all but the last token of each request (a request of one token holds nothing yet)
+    bt = random_block_tables(kv_lens, PS, n_pages, 3, "cpu")
+    kd.zero_(); vd.zero_()
+    for s, n in enumerate(kv_lens):
+        if n > 1:
+            kk, vv = _rand(n - 1, KVH * HD, dtype=dtype, seed=50 + s), _rand(n - 1, KVH * HD, dtype=dtype, seed=90 + s)
+            K.kv_write(kk.to(DEV), vv.to(DEV), kd, vd, torch.tensor(dest_for(bt, s, range(n - 1), PS), dtype=torch.int32, device=DEV), KVH, HD, PS)
+    T = len(kv_lens)
+    q = _rand(T, H * HD, dtype=dtype, seed=5).to(DEV)
+    k_new, v_new = _rand(T, KVH * HD, dtype=dtype, seed=6).to(DEV), _rand(T, KVH * HD, dtype=dtype, seed=7).to(DEV)
+    dest = torch.tensor([dest_for(bt, s, [n - 1], PS)[0] for s, n in enumerate(kv_lens)], dtype=torch.int32, device=DEV)
+    runs = [(1, n) for n in kv_lens]
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=0.2, window=window, block_tables=bt.to(DEV))
+    # the two-kernel way on a copy of the pages
+    k2, v2 = kd.clone(), vd.clone()
+    K.kv_write(k_new, v_new, k2, v2, dest, KVH, HD, PS)
+    want = torch.empty(T, H * HD, dtype=dtype, device=DEV)
+    assert K.paged_attention(q, want, k2, v2, make_meta(runs, DEV), **args) is False
+    for rep in range(2):  # twice with one workspace: the counters are left at zero
+        meta = make_meta(runs, DEV)
+        k1, v1 = kd.clone(), vd.clone()
+        got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+        assert K.paged_attention(q, got, k1, v1, meta, k_new=k_new, v_new=v_new, dest=dest, **args) is True
+        torch.testing.assert_close(got.float().cpu(), want.float().cpu(), rtol=0, atol=0)
+        torch.testing.assert_close(k1.cpu(), k2.cpu(), rtol=0, atol=0)
+        torch.testing.assert_close(v1.cpu(), v2.cpu(), rtol=0, atol=0)
+    # a launch of another shape right after, through the same workspace object
+    meta2 = make_meta(runs[:2], DEV)
+    meta2._workspaces = meta._workspaces
+    got2 = torch.empty(2, H * HD, dtype=dtype, device=DEV)
+    K.paged_attention(q[:2], got2, k2, v2, meta2, **{**args, "block_tables": bt[:2].contiguous().to(DEV)})
+    torch.testing.assert_close(got2.float().cpu(), want[:2].float().cpu(), rtol=0, atol=0)
+    # with prompt portions in the step the kernel declines and the caller writes first
+    mixed = make_meta([(2, 10), (1, 5)], DEV)
+    assert K.paged_attention(q[:3], got[:3], k2, v2, mixed, k_new=k_new[:3], v_new=v_new[:3], dest=dest[:3], **args) is False
