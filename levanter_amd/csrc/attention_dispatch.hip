@@ -8,14 +8,11 @@
 LEV_DECL(16) LEV_DECL(32) LEV_DECL(48) LEV_DECL(64) LEV_DECL(80) LEV_DECL(96) LEV_DECL(112) LEV_DECL(128)
 #undef LEV_DECL
 
-// bytes of workspace for n_decode single-token queries in `splits` splits: the counters of the (token, kv head)
-// pairs, which must be zero before the first launch (every launch leaves them zero), then the partial results
-// (the counters have a fixed place and size so that launches of different shapes can share one workspace)
-#define LEV_ATTN_COUNTERS 65536
+// bytes of workspace for the partial results of n_decode single-token queries in `splits` splits
 extern "C" long lev_attention_mfma_workspace(int n_decode, int splits, int H, int KVH, int HD) {
-  return ((long)LEV_ATTN_COUNTERS + (long)n_decode * splits * H * (HD + 2)) * (long)sizeof(float);
+  (void)KVH;
+  return (long)n_decode * splits * H * (HD + 2) * (long)sizeof(float);
 }
-extern "C" int lev_attention_mfma_max_split_rows() { return LEV_ATTN_COUNTERS; }
 
 extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
 
@@ -35,9 +32,6 @@ extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long 
   LEV_REQUIRE(n_prefill_tiles == 0 || prefill_tiles, "attention: prefill tiles are missing");
   LEV_REQUIRE(n_decode == 0 || decode_tokens, "attention: decode tokens are missing");
   LEV_REQUIRE(n_decode == 0 || splits == 1 || workspace, "attention: split decoding needs a workspace");
-  LEV_REQUIRE(splits == 1 || (long)n_decode * KVH <= LEV_ATTN_COUNTERS,
-              "attention: split decoding of %d tokens x %d kv heads exceeds the %d counters of the workspace", n_decode, KVH,
-              LEV_ATTN_COUNTERS);
   LEV_REQUIRE((k_new == nullptr) == (v_new == nullptr), "attention: new keys and values come together");
   LEV_REQUIRE(!k_new || (n_prefill_tiles == 0 && dest && kv_stride % 8 == 0 && ((uintptr_t)k_new & 15) == 0),
               "attention: new keys and values in the same launch need a step of single tokens, destinations and 16-byte aligned rows");

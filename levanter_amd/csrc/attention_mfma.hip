@@ -236,9 +236,9 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
 // ------------------------------------------------------------------------------------------------
 // Decode: one wave per (token, kv head, split). Columns of Q^T are the G = H / KVH query heads that
 // share the kv head. With more than one split the partial results go to the workspace
-//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD], counters [token][kv head]
-// and the wave that finishes last (an atomic ticket; nobody waits) merges them in the order of the
-// splits: the result does not depend on which wave that is. It resets the counter for the next launch.
+//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD]
+// and a second kernel merges them in the order of the splits. (Merging in the last wave to finish, behind an
+// atomic ticket, was measured: the device-scope fences it needs cost several times the second launch.)
 //
 // k_new != null: the step's new key and value of each token are not in the cache yet. The wave whose key
 // range holds the token's own position takes them from k_new / v_new (rows of the projection's output),
@@ -249,9 +249,8 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
                          const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
                          const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
                          const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
-                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o, int* __restrict__ counters,
+                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
                          int H, int KVH, int PS, int splits, float scale, int window) {
-  __shared__ float wz[64];
   const int lane = threadIdx.x;
   const int fr = lane & 15, g = lane >> 4;
   const int idx = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
@@ -384,41 +383,38 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(wo + 16 * dt + 4 * g) = o[dt];
   }
-  // the last wave of this (token, kv head) to get here merges the splits
-  __threadfence();  // this wave's partial results are visible to the device before its ticket is
-  int ticket = 0;
-  if (lane == 0) ticket = __hip_atomic_fetch_add(&counters[idx * KVH + kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-  ticket = __shfl(ticket, 0, 64);
-  if (ticket != splits - 1) return;
-  __threadfence();  // and the others' partial results are visible to this wave
-  if (lane == 0) counters[idx * KVH + kvh] = 0;
-  for (int hq = 0; hq < G; ++hq) {
-    const int hd_ = kvh * G + hq;
-    const size_t slot0 = ((size_t)idx * H + hd_) * splits;
-    const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
-    const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
-    const float mx = wave_max(mz);
-    const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
-    __syncthreads();  // one wave: orders the reuse of wz between heads
-    wz[lane] = w;
-    const float lsum = wave_sum(lz * w);
-    __syncthreads();
-    const float inv = 1.0f / lsum;
-    bf16_t* orow = out + (size_t)t * o_stride + (size_t)hd_ * HD;
-    for (int d = lane; d < HD; d += 64) {
-      float acc = 0.f;
-      int zz = 0;
-      for (; zz + 4 <= splits; zz += 4) {
-        const float a0 = ws_o[(slot0 + zz) * HD + d], a1 = ws_o[(slot0 + zz + 1) * HD + d];
-        const float a2 = ws_o[(slot0 + zz + 2) * HD + d], a3 = ws_o[(slot0 + zz + 3) * HD + d];
-        acc += a0 * wz[zz];
-        acc += a1 * wz[zz + 1];
-        acc += a2 * wz[zz + 2];
-        acc += a3 * wz[zz + 3];
-      }
-      for (; zz < splits; ++zz) acc += ws_o[(slot0 + zz) * HD + d] * wz[zz];
-      orow[d] = float_to_bf16(acc * inv);
+}
+
+// merge the splits of one (token, head): weights exp(m_z - max) per split, then a fixed-order sum
+__global__ void __launch_bounds__(64)
+LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __restrict__ decode_tokens,
+                          const float* __restrict__ ws_m, const float* __restrict__ ws_l, const float* __restrict__ ws_o,
+                          int H, int splits) {
+  __shared__ float wz[64];
+  const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const size_t slot0 = ((size_t)idx * H + head) * splits;
+  const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
+  const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
+  const float mx = wave_max(mz);
+  const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
+  wz[lane] = w;
+  const float l = wave_sum(lz * w);  // summed over the lanes in a fixed butterfly order
+  __syncthreads();
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + (size_t)decode_tokens[idx] * o_stride + (size_t)head * HD;
+  for (int d = lane; d < HD; d += 64) {
+    float acc = 0.f;
+    int z = 0;
+    for (; z + 4 <= splits; z += 4) {
+      const float a0 = ws_o[(slot0 + z) * HD + d], a1 = ws_o[(slot0 + z + 1) * HD + d];
+      const float a2 = ws_o[(slot0 + z + 2) * HD + d], a3 = ws_o[(slot0 + z + 3) * HD + d];
+      acc += a0 * wz[z];
+      acc += a1 * wz[z + 1];
+      acc += a2 * wz[z + 2];
+      acc += a3 * wz[z + 3];
     }
+    for (; z < splits; ++z) acc += ws_o[(slot0 + z) * HD + d] * wz[z];
+    orow[d] = float_to_bf16(acc * inv);
   }
 }
 
@@ -436,18 +432,22 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     if (int rc = lev_check_launch("attention prefill")) return rc;
   }
   if (n_decode > 0) {
-    // workspace: 65536 counters (zero between launches), then m, l, o of every (token, head, split)
+    // workspace: m, l, o of every (token, head, split)
     const size_t rows = (size_t)n_decode * H * splits;
-    int* counters = (int*)workspace;
-    float* ws_m = (float*)workspace + 65536;
+    float* ws_m = (float*)workspace;
     float* ws_l = ws_m + rows;
     float* ws_o = ws_l + rows;
     dim3 grid(n_decode, KVH, splits);
     LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages,
                                                       (bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
                                                       decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest,
-                                                      ws_m, ws_l, ws_o, counters, H, KVH, PS, splits, scale, window);
+                                                      ws_m, ws_l, ws_o, H, KVH, PS, splits, scale, window);
     if (int rc = lev_check_launch("attention decode")) return rc;
+    if (splits > 1) {
+      dim3 cgrid(n_decode, H);
+      LEV_NAME(attn_combine_hd)<<<cgrid, 64, 0, stream>>>((bf16_t*)out, o_stride, decode_tokens, ws_m, ws_l, ws_o, H, splits);
+      if (int rc = lev_check_launch("attention combine")) return rc;
+    }
   }
   return 0;
 }

@@ -191,7 +191,7 @@ class HipKernels:
         if mfma:
             splits = self.decode_splits(meta, n_heads, n_kv_heads)
             need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
-            ws = meta.zeroed_workspace(need, q.device)
+            ws = meta.workspace(need, q.device)
             self._check(self.lib.lev_attention_mfma(
                 _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles,
@@ -209,8 +209,6 @@ class HipKernels:
     def decode_splits(meta, n_heads: int, n_kv_heads: int) -> int:
         """Into how many key ranges a single-token query is split so that the chip is filled."""
         if meta.n_decode == 0:
-            return 1
-        if meta.n_decode * n_kv_heads > 65536:  # more (token, kv head) pairs than the workspace has counters: the chip is full anyway
             return 1
         want = max(1, 2048 // max(1, meta.n_decode * n_kv_heads))
         most = max(1, (meta.max_kv_len + 63) // 64)  # at least 64 keys per split

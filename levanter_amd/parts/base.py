@@ -37,15 +37,12 @@ class AttentionMeta:
     max_kv_len: int  # the longest key range any token of the step reads
     _workspaces: Dict[Any, torch.Tensor] = field(default_factory=dict)
 
-    def zeroed_workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
-        """A buffer that is zero when it is first handed out; kernels that use it leave its counters zero.
-        (``zero_()`` is a fill kernel, so this may be recorded into a graph.)"""
+    def workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
         if nbytes <= 0:
             return None
         ws = self._workspaces.get("ws")
         if ws is None or ws.numel() < nbytes:
             ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-            ws.zero_()
             self._workspaces["ws"] = ws
         return ws
 
