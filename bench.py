@@ -38,6 +38,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -97,6 +98,24 @@ def main() -> int:
         engine.reset()
         return dt, ctx_mean
 
+    def prefill_run(T, reps):
+        best = None
+        for rep in range(reps):
+            engine.reset()
+            engine.enqueue_requests([Request(prompt_tokens=prompts(1, T, 50 + rep)[0], request_id=rep, max_new_tokens=1)])
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            d = time.perf_counter() - t
+            best = d if best is None or d < best else best
+        flops = 2.0 * T * matrix_params + 2.0 * T * T * D * L + 2.0 * D * V
+        return {"value": round(T / best, 1), "tokens": T, "ms": round(best * 1e3, 3), "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_run(2048, 4)}), flush=True)
+        return 0
+
     dt, ctx_mean = decode_run(args.batch, args.steps, args.warmup, seed=1)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
@@ -116,22 +135,7 @@ def main() -> int:
     }
     if not args.no_points:
         # prefill of one 2,048-token prompt in one step (the logits of its last token)
-        T = 2048
-        best = None
-        for rep in range(3):
-            engine.reset()
-            seqs = engine.enqueue_requests([Request(prompt_tokens=prompts(1, T, 50 + rep)[0],
-                                                    request_id=rep, max_new_tokens=1)])
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            engine.step()
-            torch.cuda.synchronize()
-            d = time.perf_counter() - t
-            best = d if best is None or d < best else best
-        T_eff = T
-        flops = 2.0 * T_eff * matrix_params + 2.0 * T_eff * T_eff * D * L + 2.0 * D * V
-        out["prefill"] = {"value": round(T_eff / best, 1), "tokens": T_eff, "ms": round(best * 1e3, 3),
-                          "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
+        out["prefill"] = prefill_run(2048, 3)
         points = {}
         for b, steps in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
             d, _ = decode_run(b, steps, min(args.warmup, 4), seed=2 + b)

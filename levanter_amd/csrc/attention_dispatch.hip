@@ -1,5 +1,6 @@
 // Entry point of the matrix-core attention: checks the sizes and calls the kernels of the head size.
 #include "common.h"
+#include "attention_config.h"
 
 #define LEV_DECL(HDV)                                                                                                       \
   extern "C" int lev_attention_mfma_hd##HDV(const void*, long, void*, long, void*, void*, const int*, const int*, const int*, \
@@ -15,6 +16,9 @@ extern "C" long lev_attention_mfma_workspace(int n_decode, int splits, int H, in
 }
 
 extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
+
+// query rows of one prefill tile: the host cuts runs longer than one token into tiles of at most this many rows
+extern "C" int lev_attention_prefill_tile_rows() { return PF_ROWS; }
 
 extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long o_stride, void* k_pages, void* v_pages,
                                   const int* positions, const int* token_seq, const int* block_tables, int bt_stride,

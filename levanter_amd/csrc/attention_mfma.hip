@@ -44,36 +44,49 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   c.u = v;
   return c.b;
 }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return float2_to_bf16x2(lo, hi); }
 // key (0..63) of row i of score tile (u, h)
 __device__ __forceinline__ int tile_key(int u, int h, int i) { return 32 * u + 8 * (i >> 2) + 4 * h + (i & 3); }
 
 // One block of 64 keys for one wave: scores are in st[u][h] (S^T tiles, raw dot products).
 // Applies scale and mask, updates the running max m and sum l (per lane: column = query row),
 // rescales the output accumulators and returns the probabilities as B operands pf[u].
+// scale_log2 = scale * log2(e): scores, maxima and sums live in the base-2 domain, exp is the bare v_exp_f32.
 // q_pos: position of this lane's query row (or -1 for a padding row); key0: position of key 0 of the block.
-__device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale, int q_pos, int lo, int key0, int g, float& m,
-                                              float& l, f32x4* o, u32x4 pf[2]) {
+// need_mask (wave-uniform): false when every key of the block is visible to every row of the tile.
+__device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale_log2, int q_pos, int lo, int key0, int g,
+                                              bool need_mask, float& m, float& l, f32x4* o, u32x4 pf[2]) {
   float mx = -INFINITY;
+  if (need_mask) {
 #pragma unroll
-  for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int kp = key0 + 32 * u + 8 * g + 4 * h + r;
-        const bool ok = kp <= q_pos && kp >= lo;
-        const float s = ok ? st[u][h][r] * scale : -INFINITY;
-        st[u][h][r] = s;
-        mx = fmaxf(mx, s);
-      }
+        for (int r = 0; r < 4; ++r) {
+          const int kp = key0 + 32 * u + 8 * g + 4 * h + r;
+          const bool ok = kp <= q_pos && kp >= lo;
+          const float s = ok ? st[u][h][r] * scale_log2 : -INFINITY;
+          st[u][h][r] = s;
+          mx = fmaxf(mx, s);
+        }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float s = st[u][h][r] * scale_log2;
+          st[u][h][r] = s;
+          mx = fmaxf(mx, s);
+        }
+  }
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
   const float m_new = fmaxf(m, mx);
   const float base = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
-  const float corr = (m == -INFINITY) ? 0.f : __expf(m - base);
+  const float corr = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - base);
   float psum = 0.f;
   float p[2][2][4];
 #pragma unroll
@@ -82,7 +95,7 @@ __device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale, int q
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float e = __expf(st[u][h][r] - base);  // exp(-inf) = 0 for masked keys
+        const float e = __builtin_amdgcn_exp2f(st[u][h][r] - base);  // exp2(-inf) = 0 for masked keys
         p[u][h][r] = e;
         psum += e;
       }
@@ -99,138 +112,232 @@ __device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale, int q
 }
 
 // ------------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256)
-LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
-                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-                          const int* __restrict__ positions, const int* __restrict__ token_seq,
-                          const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int H, int KVH,
-                          int PS, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[4][NCHUNK][16][8];  // [score tile 2u+h][chunk][row][8]
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[HD][VS_STRIDE];
+// Prefill: a workgroup of PF_WAVES waves per (tile of up to PF_ROWS consecutive query tokens, head). Each wave
+// owns PF_QT tiles of 16 query rows: a key or value fragment read from LDS feeds PF_QT products, which is what
+// keeps the kernel off the LDS bandwidth limit. Blocks of 64 keys go global -> registers -> LDS; the loads of
+// the next block are in flight during the products (barriers order LDS only).
+#include "attention_config.h"
+
+typedef bf16_t (*KsPtr)[NCHUNK][16][8];
+typedef bf16_t (*VsPtr)[VS_STRIDE];
+
+__device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                                             const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+                                             const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                             const int* __restrict__ block_tables, int bt_stride, int t0, int rows, int h,
+                                             int H, int KVH, int ps_shift, float scale, int window, KsPtr Ks, VsPtr Vs) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, g = lane >> 4;
-  const int t0 = tiles[2 * blockIdx.x], rows = tiles[2 * blockIdx.x + 1];
-  const int h = blockIdx.y, kvh = h / (H / KVH);
+  const int kvh = h / (H / KVH);
+  const float scale_log2 = scale * 1.4426950408889634f;
   const int pos0 = positions[t0];
   const int* bt = block_tables + (size_t)token_seq[t0] * bt_stride;
-  const int my_row = wave * 16 + fr;
-  const int q_pos = my_row < rows ? pos0 + my_row : -1;
+  const int wave_row0 = wave * PF_QT * 16;
   const int hi = pos0 + rows - 1;                                   // last key any row needs
   const int lo_tile = window > 0 ? max(0, pos0 - window + 1) : 0;   // first key any row needs
-  const int lo = window > 0 ? max(0, q_pos - window + 1) : 0;       // first key this lane's row needs
-  const int wave_hi = min(hi, pos0 + wave * 16 + 15);
-  const bool wave_live = wave * 16 < rows;
-
-  // Q^T fragments of this lane's query row, kept for the whole kernel
-  u32x4 qf[NKS];
+  int q_pos[PF_QT], lo[PF_QT];
+  // Q^T fragments of this lane's query rows, kept for the whole kernel
+  u32x4 qf[PF_QT][NKS];
 #pragma unroll
-  for (int s = 0; s < NKS; ++s) {
-    const int c = 4 * s + g;
-    qf[s] = (q_pos >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(q + (size_t)(t0 + my_row) * q_stride + (size_t)h * HD + c * 8)
-                                        : u32x4{0, 0, 0, 0};
+  for (int qt = 0; qt < PF_QT; ++qt) {
+    const int row = wave_row0 + qt * 16 + fr;
+    q_pos[qt] = row < rows ? pos0 + row : -1;
+    lo[qt] = window > 0 ? max(0, q_pos[qt] - window + 1) : 0;
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      const int c = 4 * s + g;
+      qf[qt][s] = (q_pos[qt] >= 0 && c < NCHUNK)
+                      ? *reinterpret_cast<const u32x4*>(q + (size_t)(t0 + row) * q_stride + (size_t)h * HD + c * 8)
+                      : u32x4{0, 0, 0, 0};
+    }
   }
-  f32x4 o[NDT];
+  f32x4 o[PF_QT][NDT];
+  float m[PF_QT], l[PF_QT];
 #pragma unroll
-  for (int t = 0; t < NDT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int qt = 0; qt < PF_QT; ++qt) {
+    m[qt] = -INFINITY;
+    l[qt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) o[qt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
-  constexpr int KCH = (64 * NCHUNK + 255) / 256;  // 16-byte chunks of K per thread and block
-  constexpr int VCH = (HD * 8 + 255) / 256;
-  u32x4 kr[KCH], vr[VCH];
-  const size_t head_elems = (size_t)HD * PS;
-  auto prefetch = [&](int kb) {
+  constexpr int KCH = (64 * NCHUNK + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks of K per thread and block
+  constexpr int VCH = (HD * 8 + PF_THREADS - 1) / PF_THREADS;
+  // two register sets: block kb + 2 is loaded while block kb is multiplied (a load has two iterations to arrive)
+  u32x4 kr[2][KCH], vr[2][VCH];
+  bool kok[2][KCH], vok[2][VCH];  // does the chunk hold keys of the range (decided when it is loaded, used when it is staged)
+  const int PS = 1 << ps_shift, ps_mask = PS - 1;
+  const size_t head_elems = (size_t)HD << ps_shift;
+  // The page ids of a block of 64 keys (at most 4 of them) are read one iteration before the block's data is
+  // requested, so that no data load waits for a table lookup. They are read with vector loads on purpose (the
+  // index is made opaque): scalar loads share a counter with LDS and, while one is in flight, the compiler
+  // waits for every LDS read at once instead of pipelining them.
+  constexpr int NPG = 4;
+  // pg[0..3]: the ids as loaded (not looked at until the next iteration, so nothing waits for the loads here);
+  // pg[4]: bit j says whether entry j exists
+  auto load_pages = [&](int kb, int pg[NPG + 1]) {
+    const int b0 = (kb * 64) >> ps_shift;
+    int valid = 0;
+#pragma unroll
+    for (int j = 0; j < NPG; ++j) {
+      const int idx = b0 + j;
+      int at = min(idx, bt_stride - 1);
+      asm volatile("" : "+v"(at));
+      pg[j] = bt[at];
+      valid |= (idx < bt_stride && (j << ps_shift) < 64) ? (1 << j) : 0;
+    }
+    pg[NPG] = valid;
+  };
+  auto pick = [&](const int pg[NPG + 1], int j) {
+    const int v = j == 0 ? pg[0] : (j == 1 ? pg[1] : (j == 2 ? pg[2] : pg[3]));
+    return ((pg[NPG] >> j) & 1) ? v : -1;
+  };
+  // Loads are unconditional (a chunk outside the key range reads page 0 and is zeroed when it is staged):
+  // conditional loads would make the compiler wait for them at the join instead of after the products.
+  auto prefetch = [&](int set, int kb, const int pg[NPG + 1]) {
     const int key0 = kb * 64;
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int x = tid + 256 * i;
-      const int kk = x & 63, c = x >> 6;
+      const int x = tid + PF_THREADS * i;
+      const int kk = x & 63, c = min(x >> 6, NCHUNK - 1);
       const int kp = key0 + kk;
-      u32x4 val = u32x4{0, 0, 0, 0};
-      if (c < NCHUNK && kp <= hi && kp >= lo_tile) {
-        const int page = bt[kp / PS];
-        if (page >= 0)
-          val = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)page * KVH + kvh) * head_elems + ((size_t)c * PS + kp % PS) * 8);
-      }
-      kr[i] = val;
+      const int page = pick(pg, kk >> ps_shift);
+      kok[set][i] = kp <= hi && kp >= lo_tile && page >= 0;
+      kr[set][i] = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + (((size_t)c << ps_shift) + (kp & ps_mask)) * 8);
     }
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int y = tid + 256 * i;
+      const int y = min(tid + PF_THREADS * i, HD * 8 - 1);
       const int j = y / (HD * 2), rem = y % (HD * 2);
       const int d = rem >> 1, half = rem & 1;
-      const int kp = key0 + 16 * j + 8 * half;  // first of 8 keys; a page holds a multiple of 16
-      u32x4 val = u32x4{0, 0, 0, 0};
-      if (j < 4 && kp <= hi && kp + 7 >= lo_tile) {
-        const int page = bt[kp / PS];
-        if (page >= 0)
-          val = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)page * KVH + kvh) * head_elems + (size_t)d * PS + kp % PS);
-      }
-      vr[i] = val;
+      const int kk = 16 * j + 8 * half;  // first of 8 keys; a page holds a multiple of 16
+      const int kp = key0 + kk;
+      const int page = pick(pg, kk >> ps_shift);
+      vok[set][i] = kp <= hi && kp + 7 >= lo_tile && page >= 0;
+      vr[set][i] = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + ((size_t)d << ps_shift) + (kp & ps_mask));
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int set) {
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int x = tid + 256 * i;
+      const int x = tid + PF_THREADS * i;
       const int kk = x & 63, c = x >> 6;
       if (c < NCHUNK) {
         const int tile = 2 * (kk >> 5) + ((kk & 7) >> 2);
         const int row = 4 * ((kk & 31) >> 3) + (kk & 3);
-        *reinterpret_cast<u32x4*>(&Ks[tile][c][row][0]) = kr[i];
+        *reinterpret_cast<u32x4*>(&Ks[tile][c][row][0]) = kok[set][i] ? kr[set][i] : u32x4{0, 0, 0, 0};
       }
     }
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int y = tid + 256 * i;
-      const int j = y / (HD * 2), rem = y % (HD * 2);
-      if (j < 4) *reinterpret_cast<u32x4*>(&Vs[rem >> 1][16 * j + 8 * (rem & 1)]) = vr[i];
+      const int y = tid + PF_THREADS * i;
+      if (y < HD * 8) {
+        const int j = y / (HD * 2), rem = y % (HD * 2);
+        *reinterpret_cast<u32x4*>(&Vs[rem >> 1][16 * j + 8 * (rem & 1)]) = vok[set][i] ? vr[set][i] : u32x4{0, 0, 0, 0};
+      }
     }
   };
 
   const int kb_first = lo_tile / 64, kb_last = hi / 64;
-  prefetch(kb_first);
-  for (int kb = kb_first; kb <= kb_last; ++kb) {
-    __syncthreads();  // everyone has finished reading the previous block
-    stage();
-    __syncthreads();
-    if (kb < kb_last) prefetch(kb + 1);
+  const int n_qt = min(PF_QT, max(0, (rows - wave_row0 + 15) / 16));  // query tiles of this wave that hold rows
+  int pgs[2][NPG + 1];  // page ids of the blocks with even / odd distance from the first
+  load_pages(kb_first, pgs[0]);
+  load_pages(kb_first + 1, pgs[1]);
+  prefetch(0, kb_first, pgs[0]);
+  prefetch(1, kb_first + 1, pgs[1]);
+  load_pages(kb_first + 2, pgs[0]);
+  auto block = [&](int kb, int set) {
+    lds_barrier();  // everyone has finished reading the previous block
+    stage(set);
+    lds_barrier();
+    load_pages(kb + 3, pgs[set ^ 1]);  // older than the data loads below: waiting for them later leaves those in flight
+    prefetch(set, kb + 2, pgs[set]);   // blocks past the last one are masked by their key positions
     const int key0 = kb * 64;
-    if (!wave_live || key0 > wave_hi) continue;  // nothing in this block for this wave's rows
-    f32x4 st[2][2];
+    bool live[PF_QT];  // does query tile qt see any key of this block (wave-uniform)
+    bool any = false;
+#pragma unroll
+    for (int qt = 0; qt < PF_QT; ++qt) {
+      live[qt] = qt < n_qt && key0 <= pos0 + wave_row0 + qt * 16 + 15;
+      any = any || live[qt];
+    }
+    if (!any) return;
+    f32x4 st[PF_QT][2][2];
+#pragma unroll
+    for (int qt = 0; qt < PF_QT; ++qt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) st[qt][u][hh] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
           const int c = 4 * s + g;
           const u32x4 kf = c < NCHUNK ? *reinterpret_cast<const u32x4*>(&Ks[2 * u + hh][c][fr][0]) : u32x4{0, 0, 0, 0};
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
+#pragma unroll
+          for (int qt = 0; qt < PF_QT; ++qt)
+            if (live[qt])
+              st[qt][u][hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[qt][s]), st[qt][u][hh], 0, 0, 0);
         }
-        st[u][hh] = acc;
+    u32x4 pf[PF_QT][2];
+#pragma unroll
+    for (int qt = 0; qt < PF_QT; ++qt)
+      if (live[qt]) {
+        const int p0 = pos0 + wave_row0 + qt * 16;  // first row of the tile: does it see the whole block, and the last row too
+        const bool need_mask = !(key0 + 63 <= p0 && (window <= 0 || p0 + 15 - window + 1 <= key0));
+        softmax_block(st[qt], scale_log2, q_pos[qt], lo[qt], key0, g, need_mask, m[qt], l[qt], o[qt], pf[qt]);
       }
-    u32x4 pf[2];
-    softmax_block(st, scale, q_pos, lo, key0, g, m, l, o, pf);
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vs[16 * t + fr][32 * u + 8 * g]);
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[u]), o[t], 0, 0, 0);
-      }
-  }
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (q_pos >= 0) {
-    const float inv = 1.0f / l;
-    bf16_t* orow = out + (size_t)(t0 + my_row) * o_stride + (size_t)h * HD;
 #pragma unroll
-    for (int t = 0; t < NDT; ++t) {
-      const u32x2 v = u32x2{pack_bf16(o[t][0] * inv, o[t][1] * inv), pack_bf16(o[t][2] * inv, o[t][3] * inv)};
-      *reinterpret_cast<u32x2*>(orow + 16 * t + 4 * g) = v;
+        for (int qt = 0; qt < PF_QT; ++qt)
+          if (live[qt]) o[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[qt][u]), o[qt][t], 0, 0, 0);
+      }
+  };
+  int kb = kb_first;
+  for (; kb + 1 <= kb_last; kb += 2) {
+    block(kb, 0);
+    block(kb + 1, 1);
+  }
+  if (kb <= kb_last) block(kb, 0);
+#pragma unroll
+  for (int qt = 0; qt < PF_QT; ++qt) {
+    float lq = l[qt];
+    lq += __shfl_xor(lq, 16, 64);
+    lq += __shfl_xor(lq, 32, 64);
+    if (q_pos[qt] >= 0) {
+      const float inv = 1.0f / lq;
+      bf16_t* orow = out + (size_t)(t0 + wave_row0 + qt * 16 + fr) * o_stride + (size_t)h * HD;
+#pragma unroll
+      for (int t = 0; t < NDT; ++t) {
+        const u32x2 v = u32x2{pack_bf16(o[qt][t][0] * inv, o[qt][t][1] * inv), pack_bf16(o[qt][t][2] * inv, o[qt][t][3] * inv)};
+        *reinterpret_cast<u32x2*>(orow + 16 * t + 4 * g) = v;
+      }
     }
   }
+}
+
+// The tiles come sorted by falling number of key blocks; with `pair`, workgroup x takes tile x and then tile n - 1 - x,
+// so that every workgroup has about the same work (a causal prompt's last tile reads many times more keys than its first).
+__global__ void __launch_bounds__(PF_THREADS)
+LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+                          const int* __restrict__ positions, const int* __restrict__ token_seq,
+                          const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int n_tiles, int pair,
+                          int H, int KVH, int ps_shift, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[4][NCHUNK][16][8];  // [score tile 2u+h][chunk][row][8]
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[HD][VS_STRIDE];
+  const int first = blockIdx.x, second = n_tiles - 1 - blockIdx.x;
+  prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * first],
+               tiles[2 * first + 1], blockIdx.y, H, KVH, ps_shift, scale, window, Ks, Vs);
+  if (pair && second > first)
+    prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * second],
+                 tiles[2 * second + 1], blockIdx.y, H, KVH, ps_shift, scale, window, Ks, Vs);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -250,7 +357,9 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
                          const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
                          const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
                          float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
-                         int H, int KVH, int PS, int splits, float scale, int window) {
+                         int H, int KVH, int ps_shift, int splits, float scale, int window) {
+  const int PS = 1 << ps_shift, ps_mask = PS - 1;
+  const float scale_log2 = scale * 1.4426950408889634f;
   const int lane = threadIdx.x;
   const int fr = lane & 15, g = lane >> 4;
   const int idx = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
@@ -264,7 +373,7 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   const int kb_begin = kb_first + z * per, kb_end = min(kb_last + 1, kb_begin + per);
   const int head = kvh * G + fr;  // this lane's query head (column of Q^T)
   const int q_pos = fr < G ? pos : -1;
-  const size_t head_elems = (size_t)HD * PS;
+  const size_t head_elems = (size_t)HD << ps_shift;
   const bool fused = k_new != nullptr;
   const bool owner = fused && kb_begin <= kb_last && kb_last < kb_end;  // this wave's range holds the token's position
   const bf16_t* kn = fused ? k_new + (size_t)t * kv_stride + (size_t)kvh * HD : nullptr;
@@ -273,9 +382,9 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   if (owner) {  // the new key and value go to their page (read by later steps only)
     const int dst = dest[t];
     if (dst >= 0) {
-      bf16_t* kb_ = k_pages + ((size_t)(dst / PS) * KVH + kvh) * head_elems;
-      bf16_t* vb_ = v_pages + ((size_t)(dst / PS) * KVH + kvh) * head_elems;
-      const int off = dst % PS;
+      bf16_t* kb_ = k_pages + ((size_t)(dst >> ps_shift) * KVH + kvh) * head_elems;
+      bf16_t* vb_ = v_pages + ((size_t)(dst >> ps_shift) * KVH + kvh) * head_elems;
+      const int off = dst & ps_mask;
       for (int c = lane; c < NCHUNK; c += 64)
         *reinterpret_cast<u32x4*>(kb_ + ((size_t)c * PS + off) * 8) = *reinterpret_cast<const u32x4*>(kn + c * 8);
       for (int d = lane; d < HD; d += 64) vb_[(size_t)d * PS + off] = vn[d];
@@ -305,8 +414,8 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
         const int kp = key0 + tile_key(u, hh, fr);
         const bool ok = kp <= pos && kp >= lo;
         const bool is_new = fused && kp == pos;
-        const int page = ok ? bt[kp / PS] : -1;
-        const bf16_t* base = is_new ? kn : k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp % PS) * 8;
+        const int page = ok ? bt[kp >> ps_shift] : -1;
+        const bf16_t* base = is_new ? kn : k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp & ps_mask) * 8;
         const size_t cstride = is_new ? 8 : (size_t)PS * 8;
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
@@ -320,8 +429,8 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
     for (int u = 0; u < 2; ++u) {
       const int kp = key0 + 32 * u + 8 * g;
       const bool ok = kp <= pos && kp + 7 >= lo;
-      const int page = ok ? bt[kp / PS] : -1;
-      const bf16_t* base = v_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + kp % PS;
+      const int page = ok ? bt[kp >> ps_shift] : -1;
+      const bf16_t* base = v_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (kp & ps_mask);
       const int jn = pos - kp;  // slot of the new value among this lane's 8 keys, if 0 <= jn < 8
       const bool has_new = fused && jn >= 0 && jn < 8;
 #pragma unroll
@@ -352,7 +461,7 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
         st[u][hh] = acc;
       }
     u32x4 pf[2];
-    softmax_block(st, scale, q_pos, lo, key0, g, m, l, o, pf);
+    softmax_block(st, scale_log2, q_pos, lo, key0, g, key0 + 63 > pos || key0 < lo, m, l, o, pf);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -396,7 +505,7 @@ LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __
   const float mz = lane < splits ? ws_m[slot0 + lane] : -INFINITY;
   const float lz = lane < splits ? ws_l[slot0 + lane] : 0.f;
   const float mx = wave_max(mz);
-  const float w = mz == -INFINITY ? 0.f : __expf(mz - mx);
+  const float w = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);  // the maxima are in the base-2 domain
   wz[lane] = w;
   const float l = wave_sum(lz * w);  // summed over the lanes in a fixed butterfly order
   __syncthreads();
@@ -424,11 +533,17 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
                                                int n_prefill_tiles, const int* decode_tokens, int n_decode, const void* k_new,
                                                const void* v_new, long kv_stride, const int* dest, void* workspace, int H,
                                                int KVH, int PS, int splits, float scale, int window, hipStream_t stream) {
+  int ps_shift = 0;
+  while ((1 << ps_shift) < PS) ++ps_shift;
+  if ((1 << ps_shift) != PS) return lev_fail("attention (matrix cores): page_size=%d must be a power of two", PS);
   if (n_prefill_tiles > 0) {
-    dim3 grid(n_prefill_tiles, H);
-    LEV_NAME(attn_prefill_hd)<<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
+    // pairing halves the number of workgroups: only when every CU (256 of them) still gets one
+    const int pair = (long)n_prefill_tiles * H >= 512;
+    dim3 grid(pair ? (n_prefill_tiles + 1) / 2 : n_prefill_tiles, H);
+    LEV_NAME(attn_prefill_hd)<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
                                                         (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq,
-                                                        block_tables, bt_stride, prefill_tiles, H, KVH, PS, scale, window);
+                                                        block_tables, bt_stride, prefill_tiles, n_prefill_tiles, pair, H,
+                                                        KVH, ps_shift, scale, window);
     if (int rc = lev_check_launch("attention prefill")) return rc;
   }
   if (n_decode > 0) {
@@ -441,7 +556,7 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages,
                                                       (bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
                                                       decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest,
-                                                      ws_m, ws_l, ws_o, H, KVH, PS, splits, scale, window);
+                                                      ws_m, ws_l, ws_o, H, KVH, ps_shift, splits, scale, window);
     if (int rc = lev_check_launch("attention decode")) return rc;
     if (splits > 1) {
       dim3 cgrid(n_decode, H);

@@ -24,12 +24,19 @@ typedef uint16_t bf16_t;
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even with the hardware conversion of gfx950 (v_cvt_pk_bf16_f32); NaN stays NaN
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  union { __bf16 b; bf16_t u; } c;
+  c.b = (__bf16)f;
+  return c.u;
+}
+// two values at once: lo in the low half
+__device__ __forceinline__ uint32_t float2_to_bf16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 lev_bf16x2;
+  typedef __attribute__((ext_vector_type(2))) float lev_f32x2;
+  union { lev_bf16x2 b; uint32_t u; } c;
+  c.b = __builtin_convertvector(lev_f32x2{lo, hi}, lev_bf16x2);
+  return c.u;
 }
 
 template <typename T> __device__ __forceinline__ float to_float(T v);

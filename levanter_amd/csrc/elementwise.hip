@@ -59,8 +59,8 @@ __device__ __forceinline__ void store4<float>(float* p, float a, float b, float 
 template <>
 __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
   uint2 v;
-  v.x = (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
-  v.y = (uint32_t)float_to_bf16(c) | ((uint32_t)float_to_bf16(d) << 16);
+  v.x = float2_to_bf16x2(a, b);
+  v.y = float2_to_bf16x2(c, d);
   *reinterpret_cast<uint2*>(p) = v;
 }
 

@@ -50,8 +50,7 @@ __device__ __forceinline__ void store_vec4<float>(float* p, const float v[4]) {
 template <>
 __device__ __forceinline__ void store_vec4<bf16_t>(bf16_t* p, const float v[4]) {
   typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-  *reinterpret_cast<u32x2*>(p) = u32x2{(uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16),
-                                       (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16)};
+  *reinterpret_cast<u32x2*>(p) = u32x2{float2_to_bf16x2(v[0], v[1]), float2_to_bf16x2(v[2], v[3])};
 }
 
 template <typename TO, int BM, int BN>

@@ -84,6 +84,8 @@ class HipKernels:
             fn.restype = c_long if name.endswith("_workspace") else c_int
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
         self._sample_ws = None
+        L.lev_attention_prefill_tile_rows.restype = c_int
+        self.prefill_tile_rows = int(L.lev_attention_prefill_tile_rows())
 
     def _check(self, rc: int) -> None:
         if rc != 0:
@@ -178,7 +180,8 @@ class HipKernels:
         _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
         w = int(window) if window else 0
         qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
-        mfma = q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
+        mfma = (q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
+                and page_size & (page_size - 1) == 0)  # the matrix-core kernels index pages with shifts
         if k_new is not None:
             fusable = mfma and meta.n_prefill_tiles == 0 and meta.n_decode == T
             if not fusable:

@@ -11,9 +11,15 @@ import torch
 from levanter_amd.parts.base import AttentionMeta
 
 
-def make_meta(runs: Sequence[Tuple[int, int]], device, tile_rows: int = 64) -> AttentionMeta:
+def make_meta(runs: Sequence[Tuple[int, int]], device, tile_rows: int = 0) -> AttentionMeta:
     """runs: (q_len, kv_len after the step) per request. Tokens of a request are consecutive."""
-    positions, token_seq, tiles, decode = [], [], [], []
+    if tile_rows <= 0:
+        tile_rows = 64
+        if str(device) != "cpu":
+            from levanter_amd.kernels import get_kernels
+
+            tile_rows = get_kernels().prefill_tile_rows
+    positions, token_seq, tile_list, decode = [], [], [], []
     t0 = 0
     for s, (q_len, kv_len) in enumerate(runs):
         start = kv_len - q_len
@@ -23,8 +29,11 @@ def make_meta(runs: Sequence[Tuple[int, int]], device, tile_rows: int = 64) -> A
             decode.append(t0)
         else:
             for r0 in range(0, q_len, tile_rows):
-                tiles += [t0 + r0, min(tile_rows, q_len - r0)]
+                nr = min(tile_rows, q_len - r0)
+                tile_list.append((start + r0 + nr, t0 + r0, nr))
         t0 += q_len
+    tile_list.sort(key=lambda x: -x[0])  # falling key range, as the step function orders them
+    tiles = [v for _, first, nr in tile_list for v in (first, nr)]
 
     def dev(x):
         return torch.tensor(x, dtype=torch.int32, device=device)
