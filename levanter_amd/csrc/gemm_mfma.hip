@@ -348,11 +348,207 @@ static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const floa
 #undef LEV_SKINNY
 }
 
+// ------------------------------------------------------------------------------------------------
+// Stream kernel, for 16 < M <= 128: the weights are still the traffic that matters, but fetching the `a`
+// fragments from L2 once per wave (as the skinny kernel does) would cost more than the weights. Here a
+// workgroup of 4 waves owns 64 output columns (16 per wave) and all M rows; `a` goes through LDS in chunks of
+// 256 k and is shared by the 4 waves, each wave loads its own 16 weight rows straight into MFMA operand
+// registers. To fill the chip the K range is split over `S` workgroups (blockIdx.y); with S > 1 the partial
+// sums go to a float32 workspace [S][M][N] and a second kernel adds them in order and applies the epilogue.
+#define SK_CHUNK 64
+#define SK_LDS_STRIDE (SK_CHUNK + 8)
+
+template <typename TO, int MT>
+__global__ void __launch_bounds__(256)
+gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+                   const float* residual, long ldr, TO* out, long ldo, float* __restrict__ partial, int M, int N, int K, int act,
+                   int S) {
+  constexpr int BM = MT * 16;
+  constexpr int XCH = BM * (SK_CHUNK / 8) / 256;  // 16-byte chunks of the a tile per thread (MT = 2: 2, 4: 4, 8: 8)
+  __shared__ __attribute__((aligned(16))) bf16_t Xs[2][BM * SK_LDS_STRIDE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 15, fk = (lane >> 4) * 8;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int split = blockIdx.y;
+  const int n_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+  const int per = (n_chunks + S - 1) / S;
+  const int c_begin = split * per, c_end = min(n_chunks, c_begin + per);
+  const int n = n0 + fr;
+  const bf16_t* wrow = w + (size_t)min(n, N - 1) * K;  // a row beyond N reads the last one; its column is never stored
+  // this thread's chunks of the a tile
+  uint32_t xoff[XCH];
+  int xk[XCH], xlds[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    const int c = tid + 256 * i;
+    const int row = c / (SK_CHUNK / 8);
+    xk[i] = (c % (SK_CHUNK / 8)) * 8;
+    xoff[i] = (uint32_t)((size_t)min(row, M - 1) * lda);
+    xlds[i] = row * SK_LDS_STRIDE + xk[i];
+  }
+  u32x4 xr[XCH];
+  constexpr int KS = SK_CHUNK / 32;  // k-steps per chunk
+  u32x4 wr[2][KS];
+  auto load_x = [&](int c) {
+    const int k0 = min(c, n_chunks - 1) * SK_CHUNK;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int k = k0 + xk[i];
+      xr[i] = load16(a + xoff[i] + (k < K ? k : K - 8));
+    }
+  };
+  auto store_x = [&](int buf, int c) {
+    const int k0 = c * SK_CHUNK;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i)
+      *reinterpret_cast<u32x4*>(&Xs[buf][xlds[i]]) = (k0 + xk[i] < K) ? xr[i] : u32x4{0, 0, 0, 0};
+  };
+  auto load_w = [&](int set, int c) {
+    const int k0 = min(c, n_chunks - 1) * SK_CHUNK;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int k = k0 + s * 32 + fk;
+      wr[set][s] = load16(wrow + (k < K ? k : K - 8));  // beyond K the a fragment is zero, whatever this holds
+    }
+  };
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (c_begin < c_end) {
+    load_x(c_begin);
+    load_w(0, c_begin);
+    store_x(0, c_begin);
+    load_x(c_begin + 1);
+    load_w(1, c_begin + 1);
+    lds_barrier();
+    auto chunk = [&](int c, int set) {
+      // the a tile of chunk c + 1 (in registers since the last iteration) goes to the other buffer, then its
+      // registers and this chunk's weight registers are refilled two chunks ahead
+      const int buf = (c - c_begin) & 1;
+      store_x(buf ^ 1, c + 1);  // past this split's last chunk it fills the buffer nobody reads
+      load_x(c + 2);
+      const bf16_t* xb = &Xs[buf][fr * SK_LDS_STRIDE + fk];
+      u32x4 wcur[KS];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) wcur[s] = wr[set][s];
+      load_w(set, c + 2);
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const u32x4 af = *reinterpret_cast<const u32x4*>(xb + t * 16 * SK_LDS_STRIDE + s * 32);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(wcur[s]), acc[t], 0, 0, 0);
+        }
+      lds_barrier();
+    };
+    int c = c_begin;
+    for (; c + 1 < c_end; c += 2) {
+      chunk(c, 0);
+      chunk(c + 1, 1);
+    }
+    if (c < c_end) chunk(c, 0);
+  }
+  // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16
+  if (n < N) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = t * 16 + (lane >> 4) * 4 + r;
+        if (m < M) {
+          if (S == 1)
+            epilogue_store<TO>(acc[t][r], m, n, bias, residual, ldr, out, ldo, act);
+          else
+            partial[((size_t)split * M + m) * N + n] = acc[t][r];
+        }
+      }
+  }
+}
+
+// out = act(sum_s partial[s] + bias) + residual, the partial sums added in the order of s.
+// VEC: four consecutive columns per thread (N a multiple of 4 and every pointer and row stride aligned for it).
+template <typename TO, int VEC>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias, const float* residual, long ldr, TO* out,
+                     long ldo, int M, int N, int S, int act) {
+  const size_t total = (size_t)M * N;
+  const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * (VEC ? 4 : 1);
+  if (idx >= total) return;
+  const int m = (int)(idx / N), n = (int)(idx % N);
+  if (VEC) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(partial + idx);
+    for (int s = 1; s < S; ++s) {
+      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (size_t)s * total + idx);
+      v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+    }
+    float o[4] = {v[0], v[1], v[2], v[3]};
+    if (bias) {
+      const f32x4 b = *reinterpret_cast<const f32x4*>(bias + n);
+      o[0] += b[0]; o[1] += b[1]; o[2] += b[2]; o[3] += b[3];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = lev_activate(o[e], act);
+    if (residual) {
+      const f32x4 r = *reinterpret_cast<const f32x4*>(residual + (size_t)m * ldr + n);
+      o[0] += r[0]; o[1] += r[1]; o[2] += r[2]; o[3] += r[3];
+    }
+    store_vec4<TO>(out + (size_t)m * ldo + n, o);
+  } else {
+    float v = 0.f;
+    for (int s = 0; s < S; ++s) v += partial[(size_t)s * total + idx];
+    epilogue_store<TO>(v, m, n, bias, residual, ldr, out, ldo, act);
+  }
+}
+
+extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
+  if (M <= 16 || M > 128) return 0;
+  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+  int S = (512 + tiles - 1) / tiles;
+  if (S > chunks / 2) S = chunks / 2;
+  if (S < 1) S = 1;
+  return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
+}
+
+template <typename TO>
+static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
+                         long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
+  if ((size_t)M * lda >= (1ull << 32)) return lev_fail("linear: the activation matrix is too large (M=%d lda=%ld)", M, lda);
+  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+  int S = (512 + tiles - 1) / tiles;  // enough workgroups for two per CU
+  if (S > chunks / 2) S = chunks / 2;   // at least two chunks each
+  if (S < 1) S = 1;
+  if (S > 1 && !workspace) return lev_fail("linear: M=%d N=%d K=%d needs a workspace of lev_linear_mfma_workspace bytes", M, N, K);
+  dim3 grid(tiles, S);
+  if (M <= 32)
+    gemm_stream_kernel<TO, 2><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
+  else if (M <= 64)
+    gemm_stream_kernel<TO, 4><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
+  else
+    gemm_stream_kernel<TO, 8><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
+  if (int rc = lev_check_launch("linear_stream")) return rc;
+  if (S > 1) {
+    const size_t total = (size_t)M * N;
+    const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (((uintptr_t)workspace & 15) == 0) &&
+                     (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) && (!bias || ((uintptr_t)bias & 15) == 0);
+    if (vec)
+      splitk_reduce_kernel<TO, 1><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo,
+                                                                                            M, N, S, act);
+    else
+      splitk_reduce_kernel<TO, 0><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo, M,
+                                                                                        N, S, act);
+    return lev_check_launch("linear_reduce");
+  }
+  return 0;
+}
+
 template <typename TO>
 static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
-                             TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
-  if (M <= 64) {
+                             TO* out, long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
+  if (M <= 16) {
     launch_skinny<TO>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+  } else if (M <= 128) {
+    return launch_stream<TO>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, stream);
   } else {
     if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
       return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
@@ -372,7 +568,8 @@ static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const f
 }
 
 extern "C" int lev_linear_mfma(const void* a, long lda, const void* w, const float* bias, const float* residual, long ldr,
-                               void* out, long ldo, int M, int N, int K, int act, int out_dtype, hipStream_t stream) {
+                               void* out, long ldo, void* workspace, int M, int N, int K, int act, int out_dtype,
+                               hipStream_t stream) {
   LEV_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   LEV_REQUIRE(K % 8 == 0 && lda % 8 == 0, "linear (bfloat16): K=%d and the row stride %ld must be multiples of 8", K, lda);
   LEV_REQUIRE(((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0, "linear (bfloat16): operands must be 16-byte aligned");
@@ -381,10 +578,10 @@ extern "C" int lev_linear_mfma(const void* a, long lda, const void* w, const flo
   LEV_REQUIRE(act >= LEV_ACT_NONE && act <= LEV_ACT_TANH, "linear: unknown activation %d", act);
   if (M == 0) return 0;
   if (out_dtype == LEV_F32)
-    return linear_mfma_typed<float>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (float*)out, ldo, M, N, K,
-                                    act, stream);
+    return linear_mfma_typed<float>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (float*)out, ldo,
+                                    (float*)workspace, M, N, K, act, stream);
   if (out_dtype == LEV_BF16)
-    return linear_mfma_typed<bf16_t>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (bf16_t*)out, ldo, M, N, K,
-                                     act, stream);
+    return linear_mfma_typed<bf16_t>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (bf16_t*)out, ldo,
+                                     (float*)workspace, M, N, K, act, stream);
   return lev_fail("linear: unknown output dtype %d", out_dtype);
 }

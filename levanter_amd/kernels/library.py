@@ -72,7 +72,8 @@ class HipKernels:
             "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
             "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
             + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
-            "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 5 + [c_void_p],
+            "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p] + [c_int] * 5 + [c_void_p],
+            "lev_linear_mfma_workspace": [c_int, c_int, c_int],
             "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                    c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p]
             + [c_int] * 5 + [c_float, c_int, c_void_p],
@@ -141,7 +142,9 @@ class HipKernels:
             ldr = _rows(residual, "linear: residual")
         act = ACTIVATIONS[activation]
         if a.dtype == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
-            self._check(self.lib.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
+            need = self.lib.lev_linear_mfma_workspace(M, N, K)  # partial sums of a K range split over workgroups
+            ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need > 0 else None
+            self._check(self.lib.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
                                                  M, N, K, act, _DT[out.dtype], _stream()))
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
