@@ -1,12 +1,16 @@
 // bfloat16 matrix products on the matrix cores (MFMA), 32-bit accumulation, fused epilogue:
 //   y = act(a . w^T + bias) (+ residual),  a [M, K] (row stride lda), w [N, K], y [M, N] bf16 or f32.
-// Two kernels:
-//   tile kernel   (M > 64): 128 x 128 tile per workgroup of 4 waves, 32x32x16 MFMA, operands staged
-//                 through LDS with the next tile's global loads in flight during the products;
-//   skinny kernel (M <= 64): weight streaming. A workgroup owns 16 output columns; its waves split K,
-//                 load their part of w straight into MFMA operand registers (16x16x32), and their
-//                 partial sums are added through LDS in a fixed order (no atomics: deterministic).
-// K and lda must be multiples of 8 (16-byte operand loads); any M and N.
+// Three kernels, chosen by M:
+//   tile kernel   (M > 128): a 256x256, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
+//                 operands staged through LDS, global loads two k-tiles ahead in registers;
+//   stream kernel (16 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
+//                 straight into MFMA operand registers, K is split over workgroups and a second kernel
+//                 adds the partial sums in a fixed order;
+//   skinny kernel (M <= 16): a workgroup owns 16 output columns; its waves split K, load their part of w
+//                 straight into MFMA operand registers (16x16x32), and their partial sums are added
+//                 through LDS in a fixed order.
+// No atomics anywhere: results are deterministic. K and lda must be multiples of 8 (16-byte operand loads);
+// any M and N.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -35,7 +39,8 @@ __device__ __forceinline__ void epilogue_store(float v, int m, int n, const floa
 // Tile kernel. A workgroup of 4 waves (2 x 2) computes a BM x BN tile; a wave computes (BM/2) x (BN/2)
 // with 32x32x16 MFMA. The larger the wave's tile, the fewer LDS bytes per MFMA: 64 x 64 per wave needs
 // the whole LDS bandwidth, 128 x 128 half of it. Operand tiles of BK = 64 go global -> registers -> LDS
-// (two LDS buffers, one barrier per k-tile); the next tile's global loads are in flight during the products.
+// (two LDS buffers, one barrier per k-tile). With one wave per SIMD nothing else fills the matrix pipe
+// while a wave issues loads and LDS traffic, so those are interleaved one by one between the products.
 // Workgroups are numbered so that each XCD (id % 8) works on a contiguous band of tiles and shares
 // operands in its own L2.
 #define TK 64
@@ -69,60 +74,36 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  // XCD-aware numbering: hardware sends consecutive workgroup ids to the 8 XCDs in turn
   const int n_tiles = tiles_m * tiles_n;
   int id = blockIdx.x;
   if (n_tiles % 8 == 0) id = (id % 8) * (n_tiles / 8) + id / 8;
   const int m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
 
-  // global -> registers: rows beyond the matrix and chunks beyond K read a valid address and become zero
-  uint32_t pa[CA], pw[CW];  // element offsets of this thread's rows (the launcher checks that they fit 32 bits)
-  bool oka[CA], okw[CW];
-  int kc[CA > CW ? CA : CW];
+  // Rows beyond the matrix read the last row instead: their products land in output rows / columns that are
+  // never stored. Only the k range needs zeros, and the partial k-tile (K % 64 != 0) is taken FIRST, in the
+  // prologue, so that the main loop needs no masks at all.
+  uint32_t pa[CA], pw[CW];
+  const int kc = (tid & 7) * 8;
 #pragma unroll
-  for (int i = 0; i < CA; ++i) {
-    const int c = tid + 256 * i;
-    const int m = m0 + (c >> 3);
-    oka[i] = m < M;
-    pa[i] = (uint32_t)((size_t)(oka[i] ? m : M - 1) * lda);
-    kc[i] = (c & 7) * 8;
-  }
+  for (int i = 0; i < CA; ++i) pa[i] = (uint32_t)((size_t)min(m0 + ((tid + 256 * i) >> 3), M - 1) * lda);
 #pragma unroll
-  for (int i = 0; i < CW; ++i) {
-    const int c = tid + 256 * i;
-    const int n = n0 + (c >> 3);
-    okw[i] = n < N;
-    pw[i] = (uint32_t)((size_t)(okw[i] ? n : N - 1) * K);
-    kc[i] = (c & 7) * 8;
-  }
-  // Two register sets: while tile kt is multiplied out of LDS, the loads of tile kt + 2 are issued into one
-  // set and the other set (tile kt + 1, loaded one iteration ago) is written to the free LDS buffer between
-  // the products. A load has more than a whole iteration to arrive.
-  u32x4 ra[2][CA], rw[2][CW];
-  auto gload = [&](int set, int k0) {
-#pragma unroll
-    for (int i = 0; i < CA; ++i) {
-      const int k = k0 + kc[i];
-      ra[set][i] = load16(a + pa[i] + (k < K ? k : K - 8));  // masked when it is written to LDS: no wait for it here
-    }
-#pragma unroll
-    for (int i = 0; i < CW; ++i) {
-      const int k = k0 + kc[i];
-      rw[set][i] = load16(w + pw[i] + (k < K ? k : K - 8));
-    }
+  for (int i = 0; i < CW; ++i) pw[i] = (uint32_t)((size_t)min(n0 + ((tid + 256 * i) >> 3), N - 1) * K);
+  const int ktail = K % TK, nk = (K + TK - 1) / TK;
+  // k offset of tile t (tiles past the end repeat the last one; they are loaded but never used)
+  const int kshift = ktail ? 1 : 0;
+  auto kpos = [&](int t) {  // for t >= 1; tile 0 starts at K - ktail when there is a partial tile, else at 0
+    return max(min(t, nk - 1) - kshift, 0) * TK;
   };
-  // chunk `i` of (CA + CW) of a register set goes to LDS buffer `buf`
-  auto lstore_one = [&](int set, int buf, int k0, int i) {
-    if (i < CA) {
-      const int c = tid + 256 * i;
-      const bool ok = oka[i] && k0 + kc[i] < K;
-      *reinterpret_cast<u32x4*>(&As[buf * BM * LDS_STRIDE + (c >> 3) * LDS_STRIDE + (c & 7) * 8]) = ok ? ra[set][i] : u32x4{0, 0, 0, 0};
-    } else {
-      const int j = i - CA;
-      const int c = tid + 256 * j;
-      const bool ok = okw[j] && k0 + kc[j] < K;
-      *reinterpret_cast<u32x4*>(&Ws[buf * BN * LDS_STRIDE + (c >> 3) * LDS_STRIDE + (c & 7) * 8]) = ok ? rw[set][j] : u32x4{0, 0, 0, 0};
-    }
+  u32x4 ra[2][CA], rw[2][CW];
+  auto gload_one = [&](int set, uint32_t koff, int i) {
+    if (i < CA) ra[set][i] = load16(a + pa[i] + koff);
+    else rw[set][i - CA] = load16(w + pw[i - CA] + koff);
+  };
+  bf16_t* a_st = As + (tid >> 3) * LDS_STRIDE + kc;
+  bf16_t* w_st = Ws + (tid >> 3) * LDS_STRIDE + kc;
+  auto lstore_one = [&](int set, int buf, int i) {
+    if (i < CA) *reinterpret_cast<u32x4*>(a_st + buf * BM * LDS_STRIDE + i * 32 * LDS_STRIDE) = ra[set][i];
+    else *reinterpret_cast<u32x4*>(w_st + buf * BN * LDS_STRIDE + (i - CA) * 32 * LDS_STRIDE) = rw[set][i - CA];
   };
 
   f32x16 acc[TI][TJ];
@@ -133,31 +114,46 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = (K + TK - 1) / TK;
-  gload(0, 0);
+  {  // prologue: tile 0 (masked in k) to LDS buffer 0, tile 1 into register set 1
+    const int k0 = ktail ? K - ktail : 0;
+    const bool ok = k0 + kc < K;
+    const uint32_t koff = (uint32_t)min(k0 + kc, K - 8);
 #pragma unroll
-  for (int i = 0; i < CA + CW; ++i) lstore_one(0, 0, 0, i);
-  gload(1, min(1, nk - 1) * TK);
+    for (int i = 0; i < CA + CW; ++i) gload_one(0, koff, i);
+#pragma unroll
+    for (int i = 0; i < CA; ++i) if (!ok) ra[0][i] = u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < CW; ++i) if (!ok) rw[0][i] = u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < CA + CW; ++i) lstore_one(0, 0, i);
+    const uint32_t koff1 = (uint32_t)min(kpos(1) + kc, K - 8);
+#pragma unroll
+    for (int i = 0; i < CA + CW; ++i) gload_one(1, koff1, i);
+  }
   lds_barrier();
   const int fr = lane & 31, fk = (lane >> 5) * 8;
   constexpr int KS = TK / 16;
-  constexpr int PER = (CA + CW + KS - 1) / KS;  // LDS writes issued after each k-step's products
+  constexpr int NM = TI * TJ, NR = TI + TJ;
+  constexpr int PW = (CA + CW + KS - 2) / (KS - 1);  // LDS writes / global loads per k-step, in the first KS - 1 k-steps
+  const bf16_t* a_rd = As + (wm * WM + fr) * LDS_STRIDE + fk;
+  const bf16_t* w_rd = Ws + (wn * WN + fr) * LDS_STRIDE + fk;
+  u32x4 af[2][TI], wf[2][TJ];
+#pragma unroll
+  for (int i = 0; i < TI; ++i) af[0][i] = *reinterpret_cast<const u32x4*>(a_rd + i * 32 * LDS_STRIDE);
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) wf[0][j] = *reinterpret_cast<const u32x4*>(w_rd + j * 32 * LDS_STRIDE);
 
-  // one k-tile: `cur` is the register set that holds tile kt + 1, the other set receives tile kt + 2
+  // One k-tile. `cur` is the register set that holds tile kt + 1 (it goes to the other LDS buffer during the
+  // first KS - 1 k-steps); the other set receives the loads of tile kt + 2. Then one barrier, and the last
+  // k-step's products cover the LDS reads of tile kt + 1's first fragments. Every product is followed by at
+  // most two other instructions so that the matrix pipe never waits for the wave to issue them in a block.
   auto ktile = [&](int kt, int cur) {
     const int buf = kt & 1;
-    // always issued (past the end it re-reads the last tile, which is never stored): a conditional load would
-    // make the compiler's wait counters conservative at the join and serialise the two register sets
-    gload(cur ^ 1, min(kt + 2, nk - 1) * TK);
-    __builtin_amdgcn_sched_barrier(0);
-    const bf16_t* Ab = As + buf * BM * LDS_STRIDE + (wm * WM + fr) * LDS_STRIDE + fk;
-    const bf16_t* Wb = Ws + buf * BN * LDS_STRIDE + (wn * WN + fr) * LDS_STRIDE + fk;
-    // the fragments of k-step ks + 1 are read from LDS before the products of k-step ks are issued
-    u32x4 af[2][TI], wf[2][TJ];
-#pragma unroll
-    for (int i = 0; i < TI; ++i) af[0][i] = *reinterpret_cast<const u32x4*>(Ab + i * 32 * LDS_STRIDE);
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) wf[0][j] = *reinterpret_cast<const u32x4*>(Wb + j * 32 * LDS_STRIDE);
+    const uint32_t koff = (uint32_t)min(kpos(kt + 2) + kc, K - 8);
+    const bf16_t* Ab = a_rd + buf * BM * LDS_STRIDE;
+    const bf16_t* Wb = w_rd + buf * BN * LDS_STRIDE;
+    const bf16_t* Abn = a_rd + (buf ^ 1) * BM * LDS_STRIDE;
+    const bf16_t* Wbn = w_rd + (buf ^ 1) * BN * LDS_STRIDE;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int c = ks & 1, nx = c ^ 1;
@@ -166,19 +162,45 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
         for (int i = 0; i < TI; ++i) af[nx][i] = *reinterpret_cast<const u32x4*>(Ab + i * 32 * LDS_STRIDE + (ks + 1) * 16);
 #pragma unroll
         for (int j = 0; j < TJ; ++j) wf[nx][j] = *reinterpret_cast<const u32x4*>(Wb + j * 32 * LDS_STRIDE + (ks + 1) * 16);
+      } else {
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < TI; ++i) af[nx][i] = *reinterpret_cast<const u32x4*>(Abn + i * 32 * LDS_STRIDE);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) wf[nx][j] = *reinterpret_cast<const u32x4*>(Wbn + j * 32 * LDS_STRIDE);
       }
-      __builtin_amdgcn_sched_barrier(0);  // keep the reads of the next k-step ahead of this k-step's products
 #pragma unroll
       for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(af[c][i]), as_bf16x8(wf[c][j]), acc[i][j], 0, 0, 0);
+      if (ks + 1 < KS) {
 #pragma unroll
-      for (int q = 0; q < PER; ++q)  // after the last tile this writes the unused buffer
-        if (ks * PER + q < CA + CW) lstore_one(cur, buf ^ 1, (kt + 1) * TK, ks * PER + q);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int q = 0; q < PW; ++q)
+          if (ks * PW + q < CA + CW) lstore_one(cur, buf ^ 1, ks * PW + q);
+#pragma unroll
+        for (int q = 0; q < PW; ++q)
+          if (ks * PW + q < CA + CW) gload_one(cur ^ 1, koff, ks * PW + q);
+      }
+      constexpr int others = NR + 2 * PW;
+#pragma unroll
+      for (int m = 0; m < NM; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (ks + 1 < KS) {
+          const int lo = m * others / NM, hi = (m + 1) * others / NM;
+#pragma unroll
+          for (int o = lo; o < hi; ++o) {
+            if (o < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            else if (o < NR + PW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          }
+        } else {
+          const int lo = m * NR / NM, hi = (m + 1) * NR / NM;
+#pragma unroll
+          for (int o = lo; o < hi; ++o) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
     }
-    lds_barrier();  // not __syncthreads(): the loads of tile kt + 2 stay in flight across it
   };
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
@@ -552,13 +574,19 @@ static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const f
   } else {
     if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
       return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
-    // the largest tile that still gives every CU (256 of them) a workgroup
-    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    const long t128 = (long)((M + 255) / 256) * ((N + 127) / 128);
+    // Estimated time of each tile shape: rounds of workgroups over the 256 CUs (two 128 x 128 workgroups fit
+    // a CU) times the k-tiles plus a fixed cost for a tile's first loads and its epilogue. The constants are
+    // microseconds measured on MI355X; only their ratios matter.
+    const long nk = (K + TK - 1) / TK;
+    auto estimate = [&](int bm, int bn, long slots, double us_per_ktile) {
+      const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+      return (double)((tiles + slots - 1) / slots) * (nk * us_per_ktile + 9.0);
+    };
+    const double e256 = estimate(256, 256, 256, 2.0), e256x128 = estimate(256, 128, 256, 1.0), e128 = estimate(128, 128, 512, 1.05);
     int rc;
-    if (M > 128 && t256 >= 256)
+    if (e256 <= e256x128 && e256 <= e128)
       rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
-    else if (M > 128 && t128 >= 192)
+    else if (e256x128 <= e128)
       rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
     else
       rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
