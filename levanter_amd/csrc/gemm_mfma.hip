@@ -272,7 +272,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 // Skinny kernel. WAVES waves per workgroup; wave v takes the 32-wide k-steps v, v + WAVES, ...
 // MT = number of 16-row tiles of `a` (1..4); NT = number of 16-column tiles per workgroup (each wave
 // computes all of them from one load of its `a` fragments); U = k-steps whose loads are in flight together.
-template <typename TO, int WAVES, int MT, int NT, int U>
+template <typename TO, int WAVES, int MT, int NT, int U, int ROT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
@@ -303,14 +303,43 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // The lanes that will finish the sum fetch their bias and residual values now, so that the end of the kernel
+  // (which no other workgroup's streaming overlaps: all of them finish together) has no dependent loads left.
+  float pre_bias = 0.f;
+  f32x4 pre_res = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr bool PREFETCH_EPILOGUE = (NT * MT == 1);
+  if (PREFETCH_EPILOGUE) {
+    // unconditional loads from addresses that are always valid (clamped; `w` stands in for a missing operand):
+    // a load under a condition would make the compiler wait for it at the join, ahead of the whole k loop
+    const int nn = min(n0 + (lane & 15), N - 1);
+    const float* bp = bias ? bias + nn : reinterpret_cast<const float*>(w);
+    pre_bias = *bp;
+    if (!bias) pre_bias = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = min((lane >> 4) * 4 + r, M - 1);
+      const float* rp = residual ? residual + (size_t)m * ldr + nn : reinterpret_cast<const float*>(w);
+      pre_res[r] = *rp;
+    }
+  }
   const int nsteps = (K + 31) / 32;
+  // ROT: every workgroup starts at another place of the k range, so that they do not all read the same part
+  // of `a` and the same residue of the weight rows at the same time. The order of the sum depends on the
+  // column tile only, never on M or on what else is in the batch.
+  const int rot = ROT ? (int)((blockIdx.x * 2654435761u) % (unsigned)nsteps) : 0;
   for (int s0 = wave; s0 < nsteps; s0 += WAVES * U) {
     u32x4 wv[U][NT];
     u32x4 av[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (s0 + u * WAVES) * 32 + fk;
-      const bool k_ok = k < K;
+      int st = s0 + u * WAVES;
+      const bool s_ok = st < nsteps;
+      if (ROT) {
+        st += rot;
+        st = st >= nsteps ? st - nsteps : st;
+      }
+      const int k = st * 32 + fk;
+      const bool k_ok = s_ok && k < K;
 #pragma unroll
       for (int j = 0; j < NT; ++j) wv[u][j] = (k_ok && n_ok[j]) ? load16(wrow[j] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
@@ -343,7 +372,14 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = t * 16 + (l >> 4) * 4 + r;
-      if (m < M) epilogue_store<TO>(s[r], m, nn, bias, residual, ldr, out, ldo, act);
+      if (m >= M) continue;
+      if (PREFETCH_EPILOGUE) {  // idx == tid == lane of wave 0: the values fetched at the start
+        float v = lev_activate(s[r] + pre_bias, act);
+        if (residual) v += pre_res[r];
+        out[(size_t)m * ldo + nn] = from_float<TO>(v);
+      } else {
+        epilogue_store<TO>(s[r], m, nn, bias, residual, ldr, out, ldo, act);
+      }
     }
   }
 }
@@ -357,15 +393,15 @@ static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const floa
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
   const int mt = (M + 15) / 16;
   const int tiles = (N + 15) / 16;
-#define LEV_SKINNY(WAVES_, MT_, NT_, U_)                                                                            gemm_skinny_kernel<TO, WAVES_, MT_, NT_, U_><<<(tiles + NT_ - 1) / NT_, WAVES_ * 64, 0, stream>>>(a, lda, w, bias, residual,                                                                                                    ldr, out, ldo, M, N, K, act)
+#define LEV_SKINNY(WAVES_, MT_, NT_, U_, ROT_)                                                                            gemm_skinny_kernel<TO, WAVES_, MT_, NT_, U_, ROT_><<<(tiles + NT_ - 1) / NT_, WAVES_ * 64, 0, stream>>>(a, lda, w, bias, residual,                                                                                                    ldr, out, ldo, M, N, K, act)
   if (mt == 1) {
-    if (tiles >= 1024) LEV_SKINNY(4, 1, 1, 8); else LEV_SKINNY(8, 1, 1, 8);
+    if (tiles >= 1024) LEV_SKINNY(4, 1, 1, 8, 0); else if (tiles >= 512) LEV_SKINNY(8, 1, 1, 8, 0); else LEV_SKINNY(8, 1, 1, 4, 1);
   } else if (mt == 2) {
-    if (tiles >= 1024) LEV_SKINNY(4, 2, 1, 4); else LEV_SKINNY(8, 2, 1, 4);
+    if (tiles >= 1024) LEV_SKINNY(4, 2, 1, 4, 0); else LEV_SKINNY(8, 2, 1, 4, 0);
   } else if (tiles >= 512) {
-    if (mt == 3) LEV_SKINNY(8, 3, 2, 2); else LEV_SKINNY(8, 4, 2, 2);
+    if (mt == 3) LEV_SKINNY(8, 3, 2, 2, 0); else LEV_SKINNY(8, 4, 2, 2, 0);
   } else {
-    if (mt == 3) LEV_SKINNY(16, 3, 1, 2); else LEV_SKINNY(16, 4, 1, 2);
+    if (mt == 3) LEV_SKINNY(16, 3, 1, 2, 0); else LEV_SKINNY(16, 4, 1, 2, 0);
   }
 #undef LEV_SKINNY
 }
