@@ -165,21 +165,82 @@ extern "C" int lev_norm(const float* x, const float* w, const float* b, void* ou
 //   keys   [page][kv_head][head_dim/8][page_size][8]
 //   values [page][kv_head][head_dim][page_size]
 // dest[t] = page * page_size + offset in page; a negative dest drops the token.
+// A workgroup takes KVW_TOKENS consecutive tokens of the batch and one kv head. A key chunk of 8 elements is
+// contiguous on both sides: 16-byte (bf16) copies. Values are transposed through LDS: where 8 tokens in a row go
+// to 8 consecutive, aligned slots of one page (a prompt portion does, except at its ragged ends), a thread writes
+// its head-dim row for all 8 at once; other tokens are written element by element.
+#define KVW_TOKENS 16
+
+template <typename T>
+__device__ __forceinline__ void copy8(T* dst, const T* src) {  // 8 elements, both 16-byte aligned
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+#pragma unroll
+  for (int i = 0; i < (int)(8 * sizeof(T) / 16); ++i)
+    reinterpret_cast<u32x4*>(dst)[i] = reinterpret_cast<const u32x4*>(src)[i];
+}
+
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v, long k_stride, long v_stride,
-                                T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ dest, int KVH,
-                                int HD, int PS) {
-  const int t = blockIdx.x;
+                                T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ dest, int n_tokens,
+                                int KVH, int HD, int PS, int vec_ok) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char kvw_smem[];
+  int* dst_s = reinterpret_cast<int*>(kvw_smem);                       // [KVW_TOKENS]
+  T* vt = reinterpret_cast<T*>(kvw_smem + KVW_TOKENS * sizeof(int));   // [KVW_TOKENS][HD + 8]
+  const int ldv = HD + 8;
+  const int t0 = blockIdx.x * KVW_TOKENS;
   const int h = blockIdx.y;
-  const int dst = dest[t];
-  if (dst < 0) return;
-  const int page = dst / PS, off = dst % PS;
-  const size_t base = ((size_t)page * KVH + h) * (size_t)HD * PS;
-  const T* kr = k + (size_t)t * k_stride + (size_t)h * HD;
-  const T* vr = v + (size_t)t * v_stride + (size_t)h * HD;
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-    k_pages[base + ((size_t)(d >> 3) * PS + off) * 8 + (d & 7)] = kr[d];
-    v_pages[base + (size_t)d * PS + off] = vr[d];
+  const int tid = threadIdx.x;
+  if (tid < KVW_TOKENS) dst_s[tid] = t0 + tid < n_tokens ? dest[t0 + tid] : -1;
+  const int chunks = HD / 8;
+  // keys: one chunk of one token per thread and turn; values into LDS on the way
+  for (int idx = tid; idx < KVW_TOKENS * chunks; idx += blockDim.x) {
+    const int i = idx / chunks, c = idx % chunks;
+    const int t = t0 + i;
+    if (t >= n_tokens) continue;
+    const int dst = dest[t];
+    if (dst < 0) continue;
+    const T* kr = k + (size_t)t * k_stride + (size_t)h * HD + c * 8;
+    const T* vr = v + (size_t)t * v_stride + (size_t)h * HD + c * 8;
+    const int page = dst / PS, off = dst % PS;
+    T* kd = k_pages + ((size_t)page * KVH + h) * (size_t)HD * PS + ((size_t)c * PS + off) * 8;
+    if (vec_ok) {
+      copy8<T>(kd, kr);
+      copy8<T>(vt + i * ldv + c * 8, vr);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        kd[e] = kr[e];
+        vt[i * ldv + c * 8 + e] = vr[e];
+      }
+    }
+  }
+  __syncthreads();
+  for (int d = tid; d < HD; d += blockDim.x) {
+    int i = 0;
+    while (i < KVW_TOKENS) {
+      const int dst = dst_s[i];
+      if (dst < 0) {
+        ++i;
+        continue;
+      }
+      const int page = dst / PS, off = dst % PS;
+      T* vd = v_pages + ((size_t)page * KVH + h) * (size_t)HD * PS + (size_t)d * PS + off;
+      bool run = vec_ok && (off % 8 == 0) && i + 8 <= KVW_TOKENS;
+      if (run) {
+#pragma unroll
+        for (int j = 1; j < 8; ++j) run = run && dst_s[i + j] == dst + j;
+      }
+      if (run) {
+        __attribute__((aligned(16))) T row[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) row[j] = vt[(i + j) * ldv + d];
+        copy8<T>(vd, row);
+        i += 8;
+      } else {
+        *vd = vt[i * ldv + d];
+        ++i;
+      }
+    }
   }
 }
 
@@ -191,14 +252,20 @@ extern "C" int lev_kv_write(const void* k, const void* v, long k_stride, long v_
   LEV_REQUIRE(KVH <= 65535, "kv_write: too many kv heads (%d)", KVH);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "kv_write: unknown dtype %d", dtype);
   if (T == 0) return 0;
-  dim3 grid(T, KVH);
+  const size_t esize = dtype == LEV_F32 ? 4 : 2;
+  const size_t lds = KVW_TOKENS * sizeof(int) + (size_t)KVW_TOKENS * (HD + 8) * esize;
+  LEV_REQUIRE(lds <= 64 * 1024, "kv_write: head_dim=%d is too large", HD);
+  // 16-byte copies of the source rows need aligned rows (the pages always are: page_size and head_dim are multiples of 8)
+  const int vec_ok = ((uintptr_t)k % 16 == 0) && ((uintptr_t)v % 16 == 0) && (k_stride * esize % 16 == 0) && (v_stride * esize % 16 == 0) &&
+                     ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
+  dim3 grid((T + KVW_TOKENS - 1) / KVW_TOKENS, KVH);
   const int nt = HD <= 64 ? 64 : (HD <= 128 ? 128 : 256);
   if (dtype == LEV_F32)
-    kv_write_kernel<float><<<grid, nt, 0, stream>>>((const float*)k, (const float*)v, k_stride, v_stride, (float*)k_pages,
-                                                    (float*)v_pages, dest, KVH, HD, PS);
+    kv_write_kernel<float><<<grid, nt, lds, stream>>>((const float*)k, (const float*)v, k_stride, v_stride, (float*)k_pages,
+                                                      (float*)v_pages, dest, T, KVH, HD, PS, vec_ok);
   else
-    kv_write_kernel<bf16_t><<<grid, nt, 0, stream>>>((const bf16_t*)k, (const bf16_t*)v, k_stride, v_stride,
-                                                     (bf16_t*)k_pages, (bf16_t*)v_pages, dest, KVH, HD, PS);
+    kv_write_kernel<bf16_t><<<grid, nt, lds, stream>>>((const bf16_t*)k, (const bf16_t*)v, k_stride, v_stride,
+                                                       (bf16_t*)k_pages, (bf16_t*)v_pages, dest, T, KVH, HD, PS, vec_ok);
   return lev_check_launch("kv_write");
 }
 
