@@ -96,8 +96,9 @@ __device__ __forceinline__ void lds_barrier() {
 __device__ __forceinline__ float lev_activate(float u, int act) {
   switch (act) {
     case LEV_ACT_GELU_TANH: {
-      const float c = 0.7978845608028654f;  // sqrt(2/pi)
-      return 0.5f * u * (1.0f + tanhf(c * (u + 0.044715f * u * u * u)));
+      // 0.5 u (1 + tanh z) = u / (1 + exp(-2 z)), z = sqrt(2/pi) (u + 0.044715 u^3): no branches, unlike tanhf
+      const float c2 = 2.0f * 0.7978845608028654f;
+      return u / (1.0f + expf(-c2 * (u + 0.044715f * u * u * u)));
     }
     case LEV_ACT_GELU_ERF: return 0.5f * u * (1.0f + erff(u * 0.7071067811865476f));
     case LEV_ACT_RELU: return fmaxf(u, 0.f);
@@ -106,4 +107,10 @@ __device__ __forceinline__ float lev_activate(float u, int act) {
     case LEV_ACT_TANH: return tanhf(u);
     default: return u;
   }
+}
+
+// ACT >= 0: the activation is known at compile time (no switch per element in a hot loop); ACT < 0: `act` decides
+template <int ACT>
+__device__ __forceinline__ float lev_activate_as(float u, int act) {
+  return lev_activate(u, ACT >= 0 ? ACT : act);
 }

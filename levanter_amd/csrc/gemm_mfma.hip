@@ -58,6 +58,68 @@ __device__ __forceinline__ void store_vec4<bf16_t>(bf16_t* p, const float v[4]) 
   *reinterpret_cast<u32x2*>(p) = u32x2{float2_to_bf16x2(v[0], v[1]), float2_to_bf16x2(v[2], v[3])};
 }
 
+// Output of a wave's (TI x 32) x (TJ x 32) accumulators through an LDS area of its own: 32 rows at a time are
+// staged and written out as rows of 4 consecutive columns per lane, so that stores are wide and coalesced.
+// No barrier: LDS executes a wave's instructions in order, and a barrier that also waited for the global
+// stores (as __syncthreads() does) would expose their latency once per 32 rows.
+// 32x32 accumulator: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+template <typename TO, int ACT, int TI, int TJ>
+__device__ __forceinline__ void tile_epilogue(const f32x16 (&acc)[TI][TJ], float* Cs, int lane, int mw, int nw,
+                                              const float* __restrict__ bias, const float* residual, long ldr, TO* out,
+                                              long ldo, int M, int N, int act, int vec_ok) {
+  constexpr int WN = TJ * 32, CS = WN + 4;
+  constexpr int QUADS = WN / 4;           // groups of 4 columns in a staged row
+  constexpr int TURNS = 32 * QUADS / 64;  // per lane and 32 rows
+  constexpr int UNROLL_TURNS = ACT >= 0 ? 4 : 1;
+#pragma unroll
+  for (int i = 0; i < TI; ++i) {
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Cs[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * CS + j * 32 + (lane & 31)] = acc[i][j][r];
+#pragma unroll UNROLL_TURNS
+    for (int q = 0; q < TURNS; ++q) {  // four LDS reads in flight where the activation's code is short
+      const int idx = lane + 64 * q;
+      const int row = idx / QUADS, c4 = idx % QUADS;
+      const int m = mw + i * 32 + row;
+      const int n = nw + c4 * 4;
+      const f32x4 cv = *reinterpret_cast<const f32x4*>(&Cs[row * CS + c4 * 4]);
+      if (m >= M || n >= N) continue;
+      float v[4] = {cv[0], cv[1], cv[2], cv[3]};
+      const bool whole = vec_ok && n + 3 < N;
+      if (bias) {
+        if (whole) {
+          const f32x4 b = *reinterpret_cast<const f32x4*>(bias + n);
+          v[0] += b[0]; v[1] += b[1]; v[2] += b[2]; v[3] += b[3];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += bias[min(n + e, N - 1)];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = lev_activate_as<ACT>(v[e], act);
+      if (residual) {
+        const float* rrow = residual + (size_t)m * ldr;
+        if (whole) {
+          const f32x4 rr = *reinterpret_cast<const f32x4*>(rrow + n);
+          v[0] += rr[0]; v[1] += rr[1]; v[2] += rr[2]; v[3] += rr[3];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += rrow[min(n + e, N - 1)];
+        }
+      }
+      TO* orow = out + (size_t)m * ldo + n;
+      if (whole) {
+        store_vec4<TO>(orow, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) orow[e] = from_float<TO>(v[e]);
+      }
+    }
+  }
+}
+
 template <typename TO, int BM, int BN>
 __global__ void __launch_bounds__(256)
 gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
@@ -67,7 +129,6 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   constexpr int TI = WM / 32, TJ = WN / 32;  // in 32 x 32 MFMA tiles
   constexpr int CA = BM * (TK / 8) / 256;    // 16-byte chunks of the a tile per thread
   constexpr int CW = BN * (TK / 8) / 256;
-  constexpr int CS = WN + 4;                 // row stride (floats) of a wave's output staging area
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
   bf16_t* As = smem;                               // [2][BM * LDS_STRIDE]
   bf16_t* Ws = smem + 2 * BM * LDS_STRIDE;         // [2][BN * LDS_STRIDE]
@@ -209,42 +270,17 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   }
   if (kt < nk) ktile(kt, 1);
 
-  // Epilogue through LDS (the operand buffers are free now): each wave stages 32 rows of its tile at a time
-  // and writes them out as rows of 4 consecutive columns per lane, so that stores are wide and coalesced.
-  // 32x32 accumulator: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
-  float* Cs = reinterpret_cast<float*>(smem) + wave * 32 * CS;
-#pragma unroll
-  for (int i = 0; i < TI; ++i) {
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < TJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) Cs[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * CS + j * 32 + (lane & 31)] = acc[i][j][r];
-    __syncthreads();
-    for (int idx = lane; idx < 32 * (WN / 4); idx += 64) {
-      const int row = idx / (WN / 4), c4 = idx % (WN / 4);
-      const int m = m0 + wm * WM + i * 32 + row;
-      const int n = n0 + wn * WN + c4 * 4;
-      if (m >= M || n >= N) continue;
-      const f32x4 cv = *reinterpret_cast<const f32x4*>(&Cs[row * CS + c4 * 4]);
-      float v[4] = {cv[0], cv[1], cv[2], cv[3]};
-      if (vec_ok && n + 3 < N) {
-        if (bias) {
-          const f32x4 b = *reinterpret_cast<const f32x4*>(bias + n);
-          v[0] += b[0]; v[1] += b[1]; v[2] += b[2]; v[3] += b[3];
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = lev_activate(v[e], act);
-        if (residual) {
-          const f32x4 rr = *reinterpret_cast<const f32x4*>(residual + (size_t)m * ldr + n);
-          v[0] += rr[0]; v[1] += rr[1]; v[2] += rr[2]; v[3] += rr[3];
-        }
-        store_vec4<TO>(out + (size_t)m * ldo + n, v);
-      } else {
-        for (int e = 0; e < 4 && n + e < N; ++e) epilogue_store<TO>(v[e], m, n + e, bias, residual, ldr, out, ldo, act);
-      }
-    }
-  }
+  // Epilogue (the operand buffers are free now), specialised for the two activations that matter so that the
+  // loop over the outputs has no switch inside
+  lds_barrier();
+  float* Cs = reinterpret_cast<float*>(smem) + wave * 32 * (BN / 2 + 4);
+  const int mw = m0 + wm * WM, nw = n0 + wn * WN;
+  if (act == LEV_ACT_NONE)
+    tile_epilogue<TO, LEV_ACT_NONE, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+  else if (act == LEV_ACT_GELU_TANH)
+    tile_epilogue<TO, LEV_ACT_GELU_TANH, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+  else
+    tile_epilogue<TO, -1, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
 }
 
 template <typename TO, int BM, int BN>
