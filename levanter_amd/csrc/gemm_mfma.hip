@@ -305,141 +305,126 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel. WAVES waves per workgroup; wave v takes the 32-wide k-steps v, v + WAVES, ...
-// MT = number of 16-row tiles of `a` (1..4); NT = number of 16-column tiles per workgroup (each wave
-// computes all of them from one load of its `a` fragments); U = k-steps whose loads are in flight together.
-template <typename TO, int WAVES, int MT, int NT, int U, int ROT>
+// Skinny kernel (M <= 16). A workgroup owns 16 output columns; its WAVES waves split K. A wave takes pairs of
+// adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
+//   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
+//   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
+//            for rows 8..15 of a pair - and turned into the operand layout (row l%16, k-group l/16) through a
+//            small LDS area of the wave's own. Reading `a` in operand layout (64 bytes of each of 16 rows per
+//            instruction) costs as much time in the memory pipeline as the weights themselves: every workgroup
+//            reads all of `a`, and half lines are fetched at half the rate.
+// The partial sums of the waves are added through LDS in wave order. ROT: every workgroup starts at another
+// place of the k range, so that they do not all read the same part of `a` and the same residue of the weight
+// rows at the same time; the order of the sum depends on the column tile only, never on M or the batch.
+#define SKINNY_SLOTS 72  // 16-byte slots of one staged instruction: 8 rows x (8 chunks + 1 of padding)
+
+template <typename TO, int WAVES, int U, int ROT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
-  __shared__ f32x4 red[WAVES][NT][MT][64];
+  __shared__ f32x4 red[WAVES][64];
+  __shared__ u32x4 stage[WAVES][2][SKINNY_SLOTS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * 16 * NT;
-  const int fr = lane & 15, fk = (lane >> 4) * 8;
-  const bf16_t* wrow[NT];
-  bool n_ok[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int n = n0 + j * 16 + fr;
-    n_ok[j] = n < N;
-    wrow[j] = w + (size_t)(n_ok[j] ? n : 0) * K;
-  }
-  const bf16_t* arow[MT];
-  bool m_ok[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + fr;
-    m_ok[t] = m < M;
-    arow[t] = a + (size_t)(m_ok[t] ? m : 0) * lda;
-  }
-  f32x4 acc[NT][MT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j)
-#pragma unroll
-    for (int t = 0; t < MT; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int n0 = blockIdx.x * 16;
+  const int fr = lane & 15, kg = lane >> 4;
+  const bool n_ok = n0 + fr < N;
+  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + fr : 0) * K + kg * 8;
+  const int ar = lane >> 3, ac = lane & 7;  // `a` loads: row (0..7, second instruction +8) and chunk of the line
+  const bool a_ok0 = ar < M, a_ok1 = ar + 8 < M;
+  const bf16_t* arow0 = a + (size_t)(a_ok0 ? ar : 0) * lda + ac * 8;
+  const bf16_t* arow1 = a + (size_t)(a_ok1 ? ar + 8 : 0) * lda + ac * 8;
+  u32x4* my_stage = &stage[wave][0][0];
+  const int st_slot = ar * 9 + ac;                       // where this lane's chunk is staged
+  const int ld_slot = (fr >> 3) * SKINNY_SLOTS + (fr & 7) * 9 + kg;  // operand (row fr, k-group kg) of the pair's first step
 
   // The lanes that will finish the sum fetch their bias and residual values now, so that the end of the kernel
   // (which no other workgroup's streaming overlaps: all of them finish together) has no dependent loads left.
-  float pre_bias = 0.f;
-  f32x4 pre_res = f32x4{0.f, 0.f, 0.f, 0.f};
-  constexpr bool PREFETCH_EPILOGUE = (NT * MT == 1);
-  if (PREFETCH_EPILOGUE) {
-    // unconditional loads from addresses that are always valid (clamped; `w` stands in for a missing operand):
-    // a load under a condition would make the compiler wait for it at the join, ahead of the whole k loop
-    const int nn = min(n0 + (lane & 15), N - 1);
+  // Unconditional loads from addresses that are always valid (clamped; `w` stands in for a missing operand):
+  // a load under a condition would make the compiler wait for it at the join, ahead of the whole k loop.
+  float pre_bias;
+  f32x4 pre_res;
+  {
+    const int nn = min(n0 + fr, N - 1);
     const float* bp = bias ? bias + nn : reinterpret_cast<const float*>(w);
     pre_bias = *bp;
     if (!bias) pre_bias = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int m = min((lane >> 4) * 4 + r, M - 1);
+      const int m = min(kg * 4 + r, M - 1);
       const float* rp = residual ? residual + (size_t)m * ldr + nn : reinterpret_cast<const float*>(w);
       pre_res[r] = *rp;
     }
   }
-  const int nsteps = (K + 31) / 32;
-  // ROT: every workgroup starts at another place of the k range, so that they do not all read the same part
-  // of `a` and the same residue of the weight rows at the same time. The order of the sum depends on the
-  // column tile only, never on M or on what else is in the batch.
-  const int rot = ROT ? (int)((blockIdx.x * 2654435761u) % (unsigned)nsteps) : 0;
-  for (int s0 = wave; s0 < nsteps; s0 += WAVES * U) {
-    u32x4 wv[U][NT];
-    u32x4 av[U][MT];
+
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int npairs = (K + 63) / 64;
+  const int rot = ROT ? (int)((blockIdx.x * 2654435761u) % (unsigned)npairs) : 0;
+  for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
+    u32x4 wv[U][2], av[U][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      int st = s0 + u * WAVES;
-      const bool s_ok = st < nsteps;
+      int pr = p0 + u * WAVES;
+      const bool p_ok = pr < npairs;
       if (ROT) {
-        st += rot;
-        st = st >= nsteps ? st - nsteps : st;
+        pr += rot;
+        pr = pr >= npairs ? pr - npairs : pr;
       }
-      const int k = st * 32 + fk;
-      const bool k_ok = s_ok && k < K;
-#pragma unroll
-      for (int j = 0; j < NT; ++j) wv[u][j] = (k_ok && n_ok[j]) ? load16(wrow[j] + k) : u32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int t = 0; t < MT; ++t) av[u][t] = (k_ok && m_ok[t]) ? load16(arow[t] + k) : u32x4{0, 0, 0, 0};
+      const int k = pr * 64;
+      const bool w_ok = p_ok && n_ok;
+      wv[u][0] = (w_ok && k + kg * 8 < K) ? load16(wrow + k) : u32x4{0, 0, 0, 0};
+      wv[u][1] = (w_ok && k + 32 + kg * 8 < K) ? load16(wrow + k + 32) : u32x4{0, 0, 0, 0};
+      const bool c_ok = p_ok && k + ac * 8 < K;
+      av[u][0] = (c_ok && a_ok0) ? load16(arow0 + k) : u32x4{0, 0, 0, 0};
+      av[u][1] = (c_ok && a_ok1) ? load16(arow1 + k) : u32x4{0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av[u][t]), as_bf16x8(wv[u][j]), acc[j][t], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      // LDS executes a wave's instructions in order: the area is reused pair after pair without a barrier
+      my_stage[st_slot] = av[u][0];
+      my_stage[SKINNY_SLOTS + st_slot] = av[u][1];
+      const u32x4 a_lo = my_stage[ld_slot], a_hi = my_stage[ld_slot + 4];
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][0]), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(wv[u][1]), acc, 0, 0, 0);
+    }
   }
-#pragma unroll
-  for (int j = 0; j < NT; ++j)
-#pragma unroll
-    for (int t = 0; t < MT; ++t) red[wave][j][t][lane] = acc[j][t];
+  red[wave][lane] = acc;
   __syncthreads();
   // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16. Partial sums are added in wave order.
-  for (int idx = tid; idx < NT * MT * 64; idx += WAVES * 64) {
-    const int l = idx & 63, t = (idx >> 6) % MT, j = (idx >> 6) / MT;
-    f32x4 s = red[0][j][t][l];
+  if (wave == 0) {
+    f32x4 s = red[0][lane];
 #pragma unroll
     for (int v = 1; v < WAVES; ++v) {
-      const f32x4 o = red[v][j][t][l];
+      const f32x4 o = red[v][lane];
       s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
     }
-    const int nn = n0 + j * 16 + (l & 15);
-    if (nn >= N) continue;
+    const int nn = n0 + fr;
+    if (nn < N) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int m = t * 16 + (l >> 4) * 4 + r;
-      if (m >= M) continue;
-      if (PREFETCH_EPILOGUE) {  // idx == tid == lane of wave 0: the values fetched at the start
+      for (int r = 0; r < 4; ++r) {
+        const int m = kg * 4 + r;
+        if (m >= M) continue;
         float v = lev_activate(s[r] + pre_bias, act);
         if (residual) v += pre_res[r];
         out[(size_t)m * ldo + nn] = from_float<TO>(v);
-      } else {
-        epilogue_store<TO>(s[r], m, nn, bias, residual, ldr, out, ldo, act);
       }
     }
   }
 }
 
-// Choices measured on MI355X at K = 4096 .. 16384 (weights streamed at 4 - 6 TB/s for M <= 16):
-//   M <= 16: one column tile per workgroup, 8 loads in flight per wave;
-//   M  > 32: the `a` fragments cost more than the weights, so two column tiles share them when N is
-//            large enough to still fill the chip, and 16 waves split K when N is small.
+// Choices measured on MI355X at K = 4096 .. 16384 and M = 1 .. 16 (graph replays over distinct weights): with many
+// column tiles 4 waves with 4 or 2 pairs in flight; with fewer than 512 the chip is only filled by 16 waves per
+// workgroup. The rotated start never costs and takes a third off the time where rows are long (K = 16384).
 template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
-  const int mt = (M + 15) / 16;
   const int tiles = (N + 15) / 16;
-#define LEV_SKINNY(WAVES_, MT_, NT_, U_, ROT_)                                                                            gemm_skinny_kernel<TO, WAVES_, MT_, NT_, U_, ROT_><<<(tiles + NT_ - 1) / NT_, WAVES_ * 64, 0, stream>>>(a, lda, w, bias, residual,                                                                                                    ldr, out, ldo, M, N, K, act)
-  if (mt == 1) {
-    if (tiles >= 1024) LEV_SKINNY(4, 1, 1, 8, 0); else if (tiles >= 512) LEV_SKINNY(8, 1, 1, 8, 0); else LEV_SKINNY(8, 1, 1, 4, 1);
-  } else if (mt == 2) {
-    if (tiles >= 1024) LEV_SKINNY(4, 2, 1, 4, 0); else LEV_SKINNY(8, 2, 1, 4, 0);
-  } else if (tiles >= 512) {
-    if (mt == 3) LEV_SKINNY(8, 3, 2, 2, 0); else LEV_SKINNY(8, 4, 2, 2, 0);
-  } else {
-    if (mt == 3) LEV_SKINNY(16, 3, 1, 2, 0); else LEV_SKINNY(16, 4, 1, 2, 0);
-  }
-#undef LEV_SKINNY
+  if (tiles >= 1024)
+    gemm_skinny_kernel<TO, 4, 4, 1><<<tiles, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
+  else if (tiles >= 512)
+    gemm_skinny_kernel<TO, 4, 2, 1><<<tiles, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
+  else
+    gemm_skinny_kernel<TO, 16, 1, 1><<<tiles, 1024, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
 }
 
 // ------------------------------------------------------------------------------------------------
