@@ -1,24 +1,20 @@
-// Entry point of the matrix-core attention: checks the sizes and calls the kernels of the head size.
+// Entry point of the matrix-core attention of ONE head size (LEV_HD, one library per head size): checks the
+// sizes and calls the kernels.
 #include "common.h"
 #include "attention_config.h"
 
-#define LEV_DECL(HDV)                                                                                                       \
-  extern "C" int lev_attention_mfma_hd##HDV(const void*, long, void*, long, void*, void*, const int*, const int*, const int*, \
-                                            int, const int*, int, const int*, int, const void*, const void*, long, const int*, \
-                                            void*, int, int, int, int, float, int, hipStream_t);
-LEV_DECL(16) LEV_DECL(32) LEV_DECL(48) LEV_DECL(64) LEV_DECL(80) LEV_DECL(96) LEV_DECL(112) LEV_DECL(128)
-#undef LEV_DECL
+#ifndef LEV_HD
+#error "compile with -DLEV_HD=<head size>"
+#endif
+#define LEV_CAT2(a, b) a##b
+#define LEV_CAT(a, b) LEV_CAT2(a, b)
+#define LEV_HD_ENTRY LEV_CAT(lev_attention_mfma_hd, LEV_HD)
 
-// bytes of workspace for the partial results of n_decode single-token queries in `splits` splits
-extern "C" long lev_attention_mfma_workspace(int n_decode, int splits, int H, int KVH, int HD) {
-  (void)KVH;
-  return (long)n_decode * splits * H * (HD + 2) * (long)sizeof(float);
-}
+extern "C" int LEV_HD_ENTRY(const void*, long, void*, long, void*, void*, const int*, const int*, const int*, int, const int*, int,
+                            const int*, int, const void*, const void*, long, const int*, void*, int, int, int, int, float, int,
+                            hipStream_t);
 
-extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
-
-// query rows of one prefill tile: the host cuts runs longer than one token into tiles of at most this many rows
-extern "C" int lev_attention_prefill_tile_rows() { return PF_ROWS; }
+extern "C" int lev_attention_mfma_head_dim() { return LEV_HD; }
 
 extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long o_stride, void* k_pages, void* v_pages,
                                   const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
@@ -27,7 +23,7 @@ extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long 
                                   int KVH, int HD, int PS, int splits, float scale, int window, hipStream_t stream) {
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(H / KVH <= 16, "attention (matrix cores): at most 16 query heads per kv head, got %d", H / KVH);
-  LEV_REQUIRE(HD % 16 == 0 && HD >= 16 && HD <= 128, "attention (matrix cores): head_dim=%d must be a multiple of 16 in 16..128", HD);
+  LEV_REQUIRE(HD == LEV_HD, "attention (matrix cores): this library is built for head_dim=%d, not %d", LEV_HD, HD);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(H <= 65535 && KVH <= 65535 && splits >= 1 && splits <= 64, "attention: grid too large (heads=%d) or more than 64 splits (%d)", H, splits);
   LEV_REQUIRE(window >= 0, "attention: window=%d must not be negative", window);
@@ -39,14 +35,7 @@ extern "C" int lev_attention_mfma(const void* q, long q_stride, void* out, long 
   LEV_REQUIRE((k_new == nullptr) == (v_new == nullptr), "attention: new keys and values come together");
   LEV_REQUIRE(!k_new || (n_prefill_tiles == 0 && dest && kv_stride % 8 == 0 && ((uintptr_t)k_new & 15) == 0),
               "attention: new keys and values in the same launch need a step of single tokens, destinations and 16-byte aligned rows");
-#define LEV_CASE(HDV)                                                                                                     \
-  case HDV:                                                                                                               \
-    return lev_attention_mfma_hd##HDV(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables,    \
-                                      bt_stride, prefill_tiles, n_prefill_tiles, decode_tokens, n_decode, k_new, v_new,      \
-                                      kv_stride, dest, workspace, H, KVH, PS, splits, scale, window, stream);
-  switch (HD) {
-    LEV_CASE(16) LEV_CASE(32) LEV_CASE(48) LEV_CASE(64) LEV_CASE(80) LEV_CASE(96) LEV_CASE(112) LEV_CASE(128)
-  }
-#undef LEV_CASE
-  return lev_fail("attention (matrix cores): no kernel for head_dim=%d", HD);
+  return LEV_HD_ENTRY(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, prefill_tiles,
+                      n_prefill_tiles, decode_tokens, n_decode, k_new, v_new, kv_stride, dest, workspace, H, KVH, PS, splits, scale,
+                      window, stream);
 }

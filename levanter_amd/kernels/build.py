@@ -1,9 +1,14 @@
-"""Compiles the HIP sources under ``csrc/`` into one shared library for gfx950.
+"""Compiles the HIP sources under ``csrc/`` into shared libraries for gfx950, one per unit:
 
-The library is built in the tree (``levanter_amd/kernels/liblevanter_amd_hip.so``); when the
-tree cannot be written, in a per-user folder under the temporary directory. A build compiles
-the sources in parallel and prints a line per file, so a first call in a fresh checkout
-shows progress. ``ensure_built`` builds only when there is no library or its sources changed.
+* ``core``: errors, embedding / norms / KV write / sampling, the 32-bit GEMM and attention;
+* ``gemm_mfma``: the bfloat16 GEMMs on the matrix cores;
+* ``attn_hd<N>``: the bfloat16 attention on the matrix cores for head size N (16 .. 128 in steps of 16).
+
+A model loads ``core`` and, in bfloat16, ``gemm_mfma`` and the attention unit of its own head size, so a first
+call in a fresh checkout compiles what that model needs. The libraries are built in the tree
+(``levanter_amd/kernels/``); when the tree cannot be written, in a per-user folder under the temporary
+directory. A build compiles its sources in parallel and prints a line per file. ``ensure_built`` builds a
+unit only when it has no library or the sources changed; ``build`` builds every unit.
 """
 from __future__ import annotations
 
@@ -15,24 +20,39 @@ import sys
 import tempfile
 import time
 from concurrent.futures import ThreadPoolExecutor
-from typing import List, Optional
+from typing import Dict, Iterable, List, Optional, Tuple
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
-LIB_NAME = "liblevanter_amd_hip.so"
 ARCH = "gfx950"
 
 MFMA_ATTENTION_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
 
-# (source, extra defines, object name)
-SOURCES = [
-    ("errors.hip", [], "errors.o"),
-    ("elementwise.hip", [], "elementwise.o"),
-    ("gemm_simple.hip", [], "gemm_simple.o"),
-    ("attention_simple.hip", [], "attention_simple.o"),
-    ("gemm_mfma.hip", [], "gemm_mfma.o"),
-    ("attention_dispatch.hip", [], "attention_dispatch.o"),
-] + [("attention_mfma.hip", [f"-DLEV_HD={hd}"], f"attention_mfma_hd{hd}.o") for hd in MFMA_ATTENTION_HEAD_DIMS]
+# unit -> [(source, extra defines, object name)]
+UNITS: Dict[str, List[Tuple[str, List[str], str]]] = {
+    "core": [
+        ("errors.hip", [], "errors.o"),
+        ("elementwise.hip", [], "elementwise.o"),
+        ("gemm_simple.hip", [], "gemm_simple.o"),
+        ("attention_simple.hip", [], "attention_simple.o"),
+        ("attention_common.hip", [], "attention_common.o"),
+    ],
+    "gemm_mfma": [("gemm_mfma.hip", [], "gemm_mfma.o")],
+}
+for _hd in MFMA_ATTENTION_HEAD_DIMS:
+    UNITS[f"attn_hd{_hd}"] = [
+        ("attention_mfma.hip", [f"-DLEV_HD={_hd}"], f"attention_mfma_hd{_hd}.o"),
+        ("attention_dispatch.hip", [f"-DLEV_HD={_hd}"], f"attention_dispatch_hd{_hd}.o"),
+    ]
+
+
+def attention_unit(head_dim: int) -> str:
+    return f"attn_hd{head_dim}"
+
+
+def lib_name(unit: str) -> str:
+    return f"liblevanter_amd_{unit}.so"
+
 
 # -packed-fp32-ops off: packed 32-bit float instructions are not to be generated on this hardware pool
 HIPCC_FLAGS = [
@@ -87,16 +107,16 @@ def library_dir() -> str:
     return d
 
 
-def library_path() -> str:
-    return os.path.join(library_dir(), LIB_NAME)
+def library_path(unit: str = "core") -> str:
+    return os.path.join(library_dir(), lib_name(unit))
 
 
 def _stamp_path(lib: str) -> str:
     return lib + ".hash"
 
 
-def is_current(lib: Optional[str] = None) -> bool:
-    lib = lib or library_path()
+def is_current(unit: str = "core") -> bool:
+    lib = library_path(unit)
     try:
         with open(_stamp_path(lib)) as f:
             return os.path.isfile(lib) and f.read().strip() == source_hash()
@@ -104,25 +124,31 @@ def is_current(lib: Optional[str] = None) -> bool:
         return False
 
 
-def build(force: bool = True, jobs: Optional[int] = None) -> str:
-    """Compile every source and link the library. Returns its path."""
+def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterable[str]] = None) -> Dict[str, str]:
+    """Compile and link the given units (all of them by default). Returns unit -> library path."""
     hipcc = find_hipcc()
     if hipcc is None:
-        raise RuntimeError("hipcc not found: the HIP library of levanter_amd cannot be built (set HIPCC or install ROCm)")
-    lib = library_path()
-    if not force and is_current(lib):
-        return lib
+        raise RuntimeError("hipcc not found: the HIP libraries of levanter_amd cannot be built (set HIPCC or install ROCm)")
+    wanted = list(UNITS) if units is None else list(units)
+    for u in wanted:
+        if u not in UNITS:
+            raise RuntimeError(f"unknown kernel unit {u!r}; known: {', '.join(UNITS)}")
+    todo = [u for u in wanted if force or not is_current(u)]
+    paths = {u: library_path(u) for u in wanted}
+    if not todo:
+        return paths
     obj_dir = os.path.join(library_dir(), "_build")
     os.makedirs(obj_dir, exist_ok=True)
-    jobs = jobs or min(8, os.cpu_count() or 1, len(SOURCES))
+    items = [item for u in todo for item in UNITS[u]]
+    jobs = jobs or min(8, os.cpu_count() or 1, len(items))
     env = dict(os.environ)
     home = env.get("HOME", "")
     if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
         env["HOME"] = tempfile.gettempdir()  # hipcc wants a HOME it can write its caches to
     t0 = time.time()
-    _log(f"compiling {len(SOURCES)} HIP objects for {ARCH} with {jobs} jobs (first call only) ...")
+    _log(f"compiling {len(items)} HIP objects ({', '.join(todo)}) for {ARCH} with {jobs} jobs ...")
 
-    def compile_one(item) -> str:
+    def compile_one(item) -> None:
         src, defines, obj_name = item
         obj = os.path.join(obj_dir, obj_name)
         cmd = [hipcc, *HIPCC_FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
@@ -131,31 +157,34 @@ def build(force: bool = True, jobs: Optional[int] = None) -> str:
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src} {' '.join(defines)}:\n{_filter(r.stderr)}")
         _log(f"  {obj_name[:-2]} done in {time.time() - t:.0f}s")
-        return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs: List[str] = list(pool.map(compile_one, SOURCES))
-    tmp = lib + f".tmp{os.getpid()}"
-    r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], capture_output=True, text=True, env=env)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed to link {LIB_NAME}:\n{_filter(r.stderr)}")
-    os.replace(tmp, lib)
-    with open(_stamp_path(lib), "w") as f:
-        f.write(source_hash())
-    _log(f"built {lib} in {time.time() - t0:.0f}s")
-    return lib
+        list(pool.map(compile_one, items))
+    digest = source_hash()
+    for u in todo:
+        lib = paths[u]
+        objs = [os.path.join(obj_dir, obj_name) for _, _, obj_name in UNITS[u]]
+        tmp = lib + f".tmp{os.getpid()}"
+        r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], capture_output=True, text=True, env=env)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed to link {lib_name(u)}:\n{_filter(r.stderr)}")
+        os.replace(tmp, lib)
+        with open(_stamp_path(lib), "w") as f:
+            f.write(digest)
+    _log(f"built {', '.join(lib_name(u) for u in todo)} in {library_dir()} in {time.time() - t0:.0f}s")
+    return paths
 
 
 def _filter(stderr: str) -> str:
     return "\n".join(l for l in stderr.splitlines() if "packed-fp32-ops" not in l)
 
 
-def ensure_built() -> str:
-    """The path of a library that matches the sources; builds it if there is none."""
-    lib = library_path()
-    if is_current(lib):
+def ensure_built(unit: str = "core") -> str:
+    """The path of a library of this unit that matches the sources; builds it if there is none."""
+    lib = library_path(unit)
+    if is_current(unit):
         return lib
     if os.path.isfile(lib) and find_hipcc() is None:
         _log(f"warning: {lib} is older than its sources and hipcc is not there to rebuild it")
         return lib
-    return build(force=True)
+    return build(force=True, units=[unit])[unit]

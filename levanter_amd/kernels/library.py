@@ -55,15 +55,17 @@ def _rows(t: torch.Tensor, name: str) -> int:
 
 
 class HipKernels:
-    """The built library, loaded."""
+    """The built libraries, loaded: ``core`` at once, the bfloat16 GEMMs and the attention of a head size when a
+    call first needs them (each is compiled then, if a fresh checkout has not built it yet)."""
 
     def __init__(self, path: str):
         self.path = path
-        self.lib = ctypes.CDLL(path)
+        # RTLD_GLOBAL: the other units take the error functions (lev_fail, lev_last_error) from this library
+        self.lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
         L = self.lib
         L.lev_last_error.restype = ctypes.c_char_p
         L.lev_abi_version.restype = c_int
-        sigs = {
+        self._set_signatures(L, {
             "lev_embed": [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p],
             "lev_norm": [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_int, c_void_p],
             "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
@@ -72,21 +74,47 @@ class HipKernels:
             "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
             "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
             + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
-            "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p] + [c_int] * 5 + [c_void_p],
-            "lev_linear_mfma_workspace": [c_int, c_int, c_int],
-            "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                   c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p]
-            + [c_int] * 5 + [c_float, c_int, c_void_p],
             "lev_attention_mfma_workspace": [c_int] * 5,
-        }
-        for name, args in sigs.items():
-            fn = getattr(L, name)
-            fn.argtypes = args
-            fn.restype = c_long if name.endswith("_workspace") else c_int
+        })
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
         self._sample_ws = None
+        self._units = {}
         L.lev_attention_prefill_tile_rows.restype = c_int
         self.prefill_tile_rows = int(L.lev_attention_prefill_tile_rows())
+
+    @staticmethod
+    def _set_signatures(lib, sigs) -> None:
+        for name, args in sigs.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = c_long if name.endswith("_workspace") else c_int
+
+    def _unit(self, unit: str):
+        """The library of a unit other than ``core``, built and loaded at its first use."""
+        lib = self._units.get(unit)
+        if lib is None:
+            path = _build.ensure_built(unit)
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as e:
+                raise KernelError(f"the HIP library {path} cannot be loaded: {e}") from None
+            if unit == "gemm_mfma":
+                self._set_signatures(lib, {
+                    "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p]
+                    + [c_int] * 5 + [c_void_p],
+                    "lev_linear_mfma_workspace": [c_int, c_int, c_int],
+                })
+            else:
+                self._set_signatures(lib, {
+                    "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p]
+                    + [c_int] * 5 + [c_float, c_int, c_void_p],
+                })
+            self._units[unit] = lib
+        return lib
+
+    def loaded_units(self):
+        return ["core", *self._units]
 
     def _check(self, rc: int) -> None:
         if rc != 0:
@@ -142,9 +170,10 @@ class HipKernels:
             ldr = _rows(residual, "linear: residual")
         act = ACTIVATIONS[activation]
         if a.dtype == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
-            need = self.lib.lev_linear_mfma_workspace(M, N, K)  # partial sums of a K range split over workgroups
+            gemm = self._unit("gemm_mfma")
+            need = gemm.lev_linear_mfma_workspace(M, N, K)  # partial sums of a K range split over workgroups
             ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need > 0 else None
-            self._check(self.lib.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
+            self._check(gemm.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
                                                  M, N, K, act, _DT[out.dtype], _stream()))
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
@@ -198,7 +227,7 @@ class HipKernels:
             splits = self.decode_splits(meta, n_heads, n_kv_heads)
             need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
             ws = meta.workspace(need, q.device)
-            self._check(self.lib.lev_attention_mfma(
+            self._check(self._unit(_build.attention_unit(head_dim)).lev_attention_mfma(
                 _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles,
                 _ptr(meta.decode_tokens), meta.n_decode, _ptr(k_new), _ptr(v_new), kvs if k_new is not None else 0,
@@ -258,7 +287,7 @@ def get_kernels():
     if _KERNELS is None:
         if not torch.cuda.is_available():
             raise KernelError("levanter_amd runs on an AMD GPU only (torch.cuda.is_available() is False); there is no CPU path")
-        path = _build.ensure_built()
+        path = _build.ensure_built("core")
         try:
             _KERNELS = HipKernels(path)
         except OSError as e:
