@@ -39,6 +39,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
+    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b"],
+                    help="decode: the contract above. xl_mix / 20b: the continuous-batching workloads of BASELINE.json's configs[3] / configs[4] "
+                         "through InferenceEngine.generate; they print their own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -48,6 +51,9 @@ def main() -> int:
 
     from levanter_amd.config import InferenceEngineConfig, LmConfig
     from levanter_amd.engine import InferenceEngine, Request
+
+    if args.workload != "decode":
+        return serving_workload(args)
 
     raw = load_baseline_config()
     full_layers = raw["n_layer"]
@@ -141,6 +147,92 @@ def main() -> int:
             d, _ = decode_run(b, steps, min(args.warmup, 4), seed=2 + b)
             points[f"decode_b{b}"] = round(b * steps / d, 2)
         out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def serving_workload(args) -> int:
+    """End-to-end generation through the scheduler: requests are admitted, their prompts cut into portions under the
+    token budget beside the decoding requests, until every request has its tokens. One JSON line."""
+    import torch
+
+    from levanter_amd.config import InferenceEngineConfig, LmConfig
+    from levanter_amd.engine import InferenceEngine, Request
+
+    ps = 16
+    if args.workload == "xl_mix":  # configs[3]: gpt2_xl sizes, 64 requests, prompts U[16, 768], 128 new tokens, portions of 256
+        raw = {"model_type": "gpt2", "n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400, "vocab_size": 50257,
+               "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+        n_req, new_tokens, temperature, chunk = 64, 128, 0.0, 256
+        g = torch.Generator().manual_seed(3)
+        lens = torch.randint(16, 769, (n_req,), generator=g).tolist()
+        name = "gpt2_xl shape, 64 requests, prompts U[16,768], 128 new tokens, portions of 256"
+    else:  # configs[4]: gpt2_20b sizes, 32 requests x 1024-token prompts, 512 tokens each at temperature 1.0
+        raw = {"model_type": "gpt2", "n_layer": 44, "n_embd": 6144, "n_head": 64, "n_inner": 24576, "vocab_size": 50257,
+               "n_positions": 2048, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+        n_req, new_tokens, temperature, chunk = 32, 512, 1.0, 2048
+        lens = [1024] * n_req
+        name = "gpt2_20b shape, 32 requests x 1024-token prompts, 512 new tokens at temperature 1.0"
+    full_layers = raw["n_layer"]
+    if args.layers is not None:
+        raw["n_layer"] = args.layers
+    cfg = LmConfig.from_dict(raw)
+    V = cfg.vocab_size
+    pages_per_seq = (max(lens) + new_tokens + ps) // ps
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    if args.workload == "20b":  # the cache takes what the weights leave of the memory (a margin for activations kept)
+        free, _total = torch.cuda.mem_get_info()
+        weights = 12 * cfg.n_layer * cfg.n_embd * cfg.n_embd * itemsize + V * cfg.n_embd * itemsize
+        page_bytes = 2 * cfg.n_layer * cfg.n_embd * itemsize * ps
+        max_pages = int(max(free - weights - (24 << 30), 0) // page_bytes)
+        max_pages = max(max_pages, n_req * pages_per_seq // 2)
+    else:
+        max_pages = n_req * pages_per_seq
+    ecfg = InferenceEngineConfig(max_pages=max_pages, max_seqs=n_req, page_size=ps, max_pages_per_seq=pages_per_seq,
+                                 compute_dtype=args.dtype, max_prefill_size=chunk, max_seqs_in_prefill=n_req, seed=0)
+    t0 = time.time()
+    engine = InferenceEngine.from_config(cfg, seed=0, config=ecfg)
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f}s: {engine.model.weight_bytes() / 1e9:.2f} GB of weights, "
+          f"{max_pages} pages of {ps} tokens", file=sys.stderr, flush=True)
+
+    def requests(seed):
+        g = torch.Generator().manual_seed(seed)
+        return [Request(prompt_tokens=torch.randint(0, V, (n,), generator=g).tolist(), request_id=i, max_new_tokens=new_tokens,
+                        temperature=temperature) for i, n in enumerate(lens)]
+
+    # a short run first: kernels are loaded and the decode shapes have been seen once
+    warm = [Request(prompt_tokens=r.prompt_tokens[:32], request_id=r.request_id, max_new_tokens=4, temperature=temperature)
+            for r in requests(1)[:4]]
+    engine.generate(warm)
+    engine.reset()
+    step_ms = []
+    seqs = engine.enqueue_requests(requests(2))
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    while not all(s.done for s in seqs):
+        t1 = time.perf_counter()
+        engine.step()
+        step_ms.append((time.perf_counter() - t1) * 1e3)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t
+    generated = sum(len(s.generated) for s in seqs)
+    prompt_tokens = sum(lens)
+    step_ms.sort()
+    pick = lambda q: round(step_ms[min(len(step_ms) - 1, int(q * len(step_ms)))], 3)
+    out = {
+        "metric": f"end-to-end generated tok/s, {name}", "value": round(generated / dt, 2), "unit": "tok/s", "n_gpus": 1,
+        "steps": len(step_ms), "warmup": 0, "ms_per_step": round(dt / len(step_ms) * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
+        "config": {"model": args.workload, "n_layer": cfg.n_layer, "n_layer_full": full_layers, "n_embd": cfg.n_embd, "n_head": cfg.n_head,
+                   "head_dim": cfg.head_dim, "n_inner": cfg.inner_dim, "vocab_size": V, "n_positions": cfg.n_positions,
+                   "global_batch": n_req, "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "prefill_chunk": chunk,
+                   "page_size": ps, "max_pages": max_pages, "temperature": temperature, "parallelism": "single GPU"},
+        "seconds": round(dt, 3), "generated": generated, "all_tokens_per_s": round((generated + prompt_tokens) / dt, 1),
+        "step_ms": {"p10": pick(0.1), "p50": pick(0.5), "p90": pick(0.9), "max": round(step_ms[-1], 3)},
+        "preemptions": engine.scheduler.n_preemptions,
+    }
     print(json.dumps(out), flush=True)
     return 0
 
