@@ -103,9 +103,9 @@ class ModelRunner:
         for e in entries:
             self.cache.extend(e.handle, len(e.tokens))
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
-        batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1)
+        batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
         if graphable:
-            logits = self._run_graphed(batch)
+            logits = self._run_graphed(batch)[:batch.n_rows_real]
             if copy_out:
                 logits = logits.clone()
         else:
@@ -115,9 +115,14 @@ class ModelRunner:
         return logits
 
     # ------------------------------------------------------------------------------------
-    def _build_host(self, entries: Sequence[StepEntry], pad_blocks: int = 1) -> "HostBatch":
+    def _build_host(self, entries: Sequence[StepEntry], pad_blocks: int = 1, pad_batch: bool = False) -> "HostBatch":
         """Everything the GPU needs to know about the step, in one int32 buffer with a layout that
-        depends only on (tokens, requests, wanted rows, tiles, single tokens, blocks per request)."""
+        depends only on (tokens, requests, wanted rows, tiles, single tokens, blocks per request).
+
+        ``pad_batch`` (steps of single tokens that may be replayed as a graph): the batch is filled up to
+        ``graph_batch_bucket`` tokens with ghosts, so that a serving run whose requests end one by one meets a
+        handful of shapes instead of one per batch size. A ghost is a token 0 at position 0 that reads the first
+        request's first key, is written nowhere (destination -1) and whose logits nobody reads."""
         cache, ps = self.cache, self.cache.page_size
         S = len(entries)
         T = sum(len(e.tokens) for e in entries)
@@ -148,6 +153,18 @@ class ModelRunner:
             first_positions.append(start)
             max_blocks = max(max_blocks, (start + n + ps - 1) // ps)
             t0 += n
+        n_real_tokens, n_rows_real = T, len(rows)
+        if pad_batch and rows:
+            ghosts = graph_batch_bucket(T) - T
+            if ghosts > 0:
+                tokens = np.concatenate([tokens, np.zeros(ghosts, np.int32)])
+                positions = np.concatenate([positions, np.zeros(ghosts, np.int32)])
+                token_seq = np.concatenate([token_seq, np.zeros(ghosts, np.int32)])
+                seq_slots = np.concatenate([seq_slots, np.full(ghosts, seq_slots[0], np.int32)])
+                decode.extend(range(T, T + ghosts))
+                rows.extend([rows[0]] * ghosts)
+                S += ghosts
+                T += ghosts
         # the attention kernel pairs tile i with tile n - 1 - i: sorted by falling key range, pairs have equal work
         tile_list.sort(key=lambda x: -x[0])
         tiles: List[int] = [v for _, first, nr in tile_list for v in (first, nr)]
@@ -163,11 +180,14 @@ class ModelRunner:
             bt = g.block_tables[seq_slots, :max_blocks]
             host[offs[7 + 2 * gi]:offs[7 + 2 * gi] + S * max_blocks] = bt.reshape(-1)
             pages = g.block_tables[seq_slots[token_seq], positions // ps]
-            assert (pages != NO_PAGE).all(), "a new token has no page"
-            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = pages * ps + positions % ps
+            assert (pages[:n_real_tokens] != NO_PAGE).all(), "a new token has no page"
+            dest = pages * ps + positions % ps
+            dest[n_real_tokens:] = -1  # ghosts are written nowhere
+            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = dest
         return HostBatch(host=host, sizes=sizes, offs=[int(o) for o in offs], n_tokens=T, n_seqs=S, n_rows=len(rows),
                          n_tiles=len(tiles) // 2, n_decode=len(decode), max_blocks=max_blocks, max_kv=max_blocks * ps,
-                         run_lengths=run_lengths, first_positions=first_positions, slots=[int(x) for x in seq_slots])
+                         run_lengths=run_lengths, first_positions=first_positions, slots=[int(x) for x in seq_slots[:len(entries)]],
+                         n_rows_real=n_rows_real)
 
     def _make_ctx(self, dev: torch.Tensor, b: "HostBatch", workspaces: Dict[object, torch.Tensor]) -> StepContext:
         def view(i):
@@ -238,6 +258,12 @@ GRAPH_BLOCK_BUCKET = 16  # block tables of graphed steps are padded to a multipl
 MAX_GRAPHS = 48
 
 
+def graph_batch_bucket(n: int) -> int:
+    """Batch size that a graphed step of ``n`` single tokens is filled up to: small batches stay as they are,
+    larger ones go to the next multiple of 8 (the GEMM kernels work on row tiles of 16 anyway)."""
+    return n if n <= 4 else (n + 7) // 8 * 8
+
+
 @dataclass
 class _Graph:
     static: torch.Tensor
@@ -262,4 +288,5 @@ class HostBatch:
     run_lengths: List[int]
     first_positions: List[int]
     slots: List[int]
+    n_rows_real: int = 0
     rows_view: Optional[torch.Tensor] = None

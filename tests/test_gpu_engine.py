@@ -452,3 +452,49 @@ def test_decode_steps_replayed_from_a_hip_graph_equal_eager_steps(dtype, monkeyp
     graphs = [v for v in runners[0][0]._graphs.values() if v != "seen"]
     assert len(graphs) >= 2  # the block-table bucket changed at least once while decoding 60 tokens
     assert all(r.cache.groups[0].pool.n_free < 40 for r, _ in runners)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graphed_decode_batches_are_filled_up_with_ghost_tokens(dtype):
+    """Requests end one by one: 7, 6 and 5 live requests all run the graph of 8 rows, the missing ones being ghost
+    tokens that are written nowhere. Every step equals the same step run eagerly without ghosts (32-bit: bit for
+    bit; bfloat16: up to the rounding of another split of the key range), and the caches stay equal afterwards."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import load_model, make_cache
+    from levanter_amd.engine.step import graph_batch_bucket
+
+    assert [graph_batch_bucket(n) for n in (1, 4, 5, 8, 9, 63)] == [1, 4, 8, 8, 16, 64]
+    d = write_model(TINY_A, 0, torch.float32 if dtype == "float32" else torch.bfloat16)
+    env = _env(dtype)
+    _, model = load_model(d, env)
+    cfg = InferenceEngineConfig(max_pages=64, max_seqs=8, page_size=16, max_pages_per_seq=8, compute_dtype=dtype)
+    runners = []
+    for graphs in (True, False):
+        cache = make_cache(model, cfg)
+        runners.append((ModelRunner(model, cache, env, use_graphs=graphs), cache))
+    g = torch.Generator().manual_seed(11)
+    names = "abcdefg"
+    toks = {k: torch.randint(0, 512, (60,), generator=g).tolist() for k in names}
+    handles = [{k: c.open(k) for k in names} for _, c in runners]
+    for (r, _), h in zip(runners, handles):
+        r.step([StepEntry(h[k], toks[k][:3 + 2 * i], []) for i, k in enumerate(names)])
+    live = list(names)
+    tol = dict(rtol=0, atol=0) if dtype == "float32" else dict(rtol=2e-2, atol=8e-3)
+    for i in range(30):
+        if i in (10, 20):  # a request ends: the batch shrinks, the graph does not change
+            gone = live.pop(2)
+            for (_, c), h in zip(runners, handles):
+                c.close(h[gone])
+        outs = []
+        for (r, _), h in zip(runners, handles):
+            outs.append(r.step([StepEntry(h[k], [toks[k][h[k].length]], [0]) for k in live]).cpu())
+        assert outs[0].shape == (len(live), 512)
+        torch.testing.assert_close(outs[0], outs[1], **tol)
+    keys = [k for k, v in runners[0][0]._graphs.items() if v != "seen"]
+    assert keys and all(k[0] == 8 and k[1] == 8 for k in keys)
+    # what the steps wrote is the same with and without ghosts: one more whole-prompt-like step reads it all back
+    last = []
+    for (r, _), h in zip(runners, handles):
+        last.append(r.step([StepEntry(h[k], toks[k][h[k].length:h[k].length + 3], [2]) for k in live]).cpu())
+    torch.testing.assert_close(last[0], last[1], **tol)
