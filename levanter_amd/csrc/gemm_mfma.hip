@@ -3,10 +3,10 @@
 // Three kernels, chosen by M:
 //   tile kernel   (M > 128): a 256x256, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 operands staged through LDS, global loads two k-tiles ahead in registers;
-//   stream kernel (16 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
+//   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
 //                 straight into MFMA operand registers, K is split over workgroups and a second kernel
 //                 adds the partial sums in a fixed order;
-//   skinny kernel (M <= 16): a workgroup owns 16 output columns; its waves split K, load their part of w
+//   skinny kernel (M <= 24): a workgroup owns 16 output columns; its waves split K, load their part of w
 //                 straight into MFMA operand registers (16x16x32), and their partial sums are added
 //                 through LDS in a fixed order.
 // No atomics anywhere: results are deterministic. K and lda must be multiples of 8 (16-byte operand loads);
@@ -305,7 +305,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel (M <= 16). A workgroup owns 16 output columns; its WAVES waves split K. A wave takes pairs of
+// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns 16 output columns; its WAVES waves split K. A wave takes pairs of
 // adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
 //   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
 //   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
@@ -317,23 +317,29 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 // place of the k range, so that they do not all read the same part of `a` and the same residue of the weight
 // rows at the same time; the order of the sum depends on the column tile only, never on M or the batch.
 #define SKINNY_SLOTS 72  // 16-byte slots of one staged instruction: 8 rows x (8 chunks + 1 of padding)
+#define SKINNY_MAX_M 24  // measured: with two row tiles it beats the stream kernel up to here, at 32 rows no longer
 
-template <typename TO, int WAVES, int U, int ROT>
+template <typename TO, int WAVES, int U, int ROT, int MT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
-  __shared__ f32x4 red[WAVES][64];
-  __shared__ u32x4 stage[WAVES][2][SKINNY_SLOTS];
+  constexpr int AI = 2 * MT;  // `a` instructions per pair of k-steps: 8 rows each
+  __shared__ f32x4 red[WAVES][MT][64];
+  __shared__ u32x4 stage[WAVES][AI][SKINNY_SLOTS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * 16;
   const int fr = lane & 15, kg = lane >> 4;
   const bool n_ok = n0 + fr < N;
   const bf16_t* wrow = w + (size_t)(n_ok ? n0 + fr : 0) * K + kg * 8;
-  const int ar = lane >> 3, ac = lane & 7;  // `a` loads: row (0..7, second instruction +8) and chunk of the line
-  const bool a_ok0 = ar < M, a_ok1 = ar + 8 < M;
-  const bf16_t* arow0 = a + (size_t)(a_ok0 ? ar : 0) * lda + ac * 8;
-  const bf16_t* arow1 = a + (size_t)(a_ok1 ? ar + 8 : 0) * lda + ac * 8;
+  const int ar = lane >> 3, ac = lane & 7;  // `a` loads: row (0..7, instruction i adds 8 i) and chunk of the line
+  bool a_ok[AI];
+  const bf16_t* arow[AI];
+#pragma unroll
+  for (int i = 0; i < AI; ++i) {
+    a_ok[i] = ar + 8 * i < M;
+    arow[i] = a + (size_t)(a_ok[i] ? ar + 8 * i : 0) * lda + ac * 8;
+  }
   u32x4* my_stage = &stage[wave][0][0];
   const int st_slot = ar * 9 + ac;                       // where this lane's chunk is staged
   const int ld_slot = (fr >> 3) * SKINNY_SLOTS + (fr & 7) * 9 + kg;  // operand (row fr, k-group kg) of the pair's first step
@@ -343,25 +349,29 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   // Unconditional loads from addresses that are always valid (clamped; `w` stands in for a missing operand):
   // a load under a condition would make the compiler wait for it at the join, ahead of the whole k loop.
   float pre_bias;
-  f32x4 pre_res;
+  f32x4 pre_res[MT];
   {
     const int nn = min(n0 + fr, N - 1);
     const float* bp = bias ? bias + nn : reinterpret_cast<const float*>(w);
     pre_bias = *bp;
     if (!bias) pre_bias = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int m = min(kg * 4 + r, M - 1);
-      const float* rp = residual ? residual + (size_t)m * ldr + nn : reinterpret_cast<const float*>(w);
-      pre_res[r] = *rp;
-    }
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = min(t * 16 + kg * 4 + r, M - 1);
+        const float* rp = residual ? residual + (size_t)m * ldr + nn : reinterpret_cast<const float*>(w);
+        pre_res[t][r] = *rp;
+      }
   }
 
-  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int npairs = (K + 63) / 64;
   const int rot = ROT ? (int)((blockIdx.x * 2654435761u) % (unsigned)npairs) : 0;
   for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
-    u32x4 wv[U][2], av[U][2];
+    u32x4 wv[U][2], av[U][AI];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int pr = p0 + u * WAVES;
@@ -375,38 +385,45 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
       wv[u][0] = (w_ok && k + kg * 8 < K) ? load16(wrow + k) : u32x4{0, 0, 0, 0};
       wv[u][1] = (w_ok && k + 32 + kg * 8 < K) ? load16(wrow + k + 32) : u32x4{0, 0, 0, 0};
       const bool c_ok = p_ok && k + ac * 8 < K;
-      av[u][0] = (c_ok && a_ok0) ? load16(arow0 + k) : u32x4{0, 0, 0, 0};
-      av[u][1] = (c_ok && a_ok1) ? load16(arow1 + k) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < AI; ++i) av[u][i] = (c_ok && a_ok[i]) ? load16(arow[i] + k) : u32x4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // LDS executes a wave's instructions in order: the area is reused pair after pair without a barrier
-      my_stage[st_slot] = av[u][0];
-      my_stage[SKINNY_SLOTS + st_slot] = av[u][1];
-      const u32x4 a_lo = my_stage[ld_slot], a_hi = my_stage[ld_slot + 4];
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][0]), acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(wv[u][1]), acc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < AI; ++i) my_stage[i * SKINNY_SLOTS + st_slot] = av[u][i];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const u32x4 a_lo = my_stage[2 * t * SKINNY_SLOTS + ld_slot], a_hi = my_stage[2 * t * SKINNY_SLOTS + ld_slot + 4];
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][0]), acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(wv[u][1]), acc[t], 0, 0, 0);
+      }
     }
   }
-  red[wave][lane] = acc;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
   __syncthreads();
   // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16. Partial sums are added in wave order.
   if (wave == 0) {
-    f32x4 s = red[0][lane];
-#pragma unroll
-    for (int v = 1; v < WAVES; ++v) {
-      const f32x4 o = red[v][lane];
-      s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
-    }
     const int nn = n0 + fr;
-    if (nn < N) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = kg * 4 + r;
-        if (m >= M) continue;
-        float v = lev_activate(s[r] + pre_bias, act);
-        if (residual) v += pre_res[r];
-        out[(size_t)m * ldo + nn] = from_float<TO>(v);
+    for (int t = 0; t < MT; ++t) {
+      f32x4 s = red[0][t][lane];
+#pragma unroll
+      for (int v = 1; v < WAVES; ++v) {
+        const f32x4 o = red[v][t][lane];
+        s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
+      }
+      if (nn < N) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = t * 16 + kg * 4 + r;
+          if (m >= M) continue;
+          float v = lev_activate(s[r] + pre_bias, act);
+          if (residual) v += pre_res[t][r];
+          out[(size_t)m * ldo + nn] = from_float<TO>(v);
+        }
       }
     }
   }
@@ -419,16 +436,17 @@ template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
   const int tiles = (N + 15) / 16;
-  if (tiles >= 1024)
-    gemm_skinny_kernel<TO, 4, 4, 1><<<tiles, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
-  else if (tiles >= 512)
-    gemm_skinny_kernel<TO, 4, 2, 1><<<tiles, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
-  else
-    gemm_skinny_kernel<TO, 16, 1, 1><<<tiles, 1024, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act);
+#define LEV_SKINNY(W_, U_, MT_) gemm_skinny_kernel<TO, W_, U_, 1, MT_><<<tiles, W_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act)
+  if (M <= 16) {
+    if (tiles >= 1024) LEV_SKINNY(4, 4, 1); else if (tiles >= 512) LEV_SKINNY(4, 2, 1); else LEV_SKINNY(16, 1, 1);
+  } else {  // 17 .. SKINNY_MAX_M rows: two row tiles share every weight load
+    if (tiles >= 1024) LEV_SKINNY(4, 2, 2); else if (tiles >= 512) LEV_SKINNY(4, 2, 2); else LEV_SKINNY(16, 1, 2);
+  }
+#undef LEV_SKINNY
 }
 
 // ------------------------------------------------------------------------------------------------
-// Stream kernel, for 16 < M <= 128: the weights are still the traffic that matters, but fetching the `a`
+// Stream kernel, for 24 < M <= 128: the weights are still the traffic that matters, but fetching the `a`
 // fragments from L2 once per wave (as the skinny kernel does) would cost more than the weights. Here a
 // workgroup of 4 waves owns 64 output columns (16 per wave) and all M rows; `a` goes through LDS in chunks of
 // 256 k and is shared by the 4 waves, each wave loads its own 16 weight rows straight into MFMA operand
@@ -581,7 +599,7 @@ splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict_
 }
 
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
-  if (M <= 16 || M > 128) return 0;
+  if (M <= SKINNY_MAX_M || M > 128) return 0;
   const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
   int S = (512 + tiles - 1) / tiles;
   if (S > chunks / 2) S = chunks / 2;
@@ -624,7 +642,7 @@ static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float
 template <typename TO>
 static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                              TO* out, long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
-  if (M <= 16) {
+  if (M <= SKINNY_MAX_M) {
     launch_skinny<TO>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
   } else if (M <= 128) {
     return launch_stream<TO>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, stream);

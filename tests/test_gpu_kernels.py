@@ -77,11 +77,11 @@ def test_norm_constant_row_gives_bias(K):
     torch.testing.assert_close(got.cpu(), b.expand(2, 96), rtol=0, atol=1e-6)
 
 
-# M <= 16: weight-streaming kernel (its three launch shapes by N: 16, 4 and 4 waves; K with and without a partial
-# pair of k-steps; rows 8..15); 17..128: split-K kernel; above: tile kernels (the last shape takes 256 x 256 tiles
+# M <= 24: weight-streaming kernel (its three launch shapes by N: 16, 4 and 4 waves; K with and without a partial
+# pair of k-steps; rows 8..15; two row tiles above 16 rows); 25..128: split-K kernel; above: tile kernels (the last shape takes 256 x 256 tiles
 # and a partial k-tile)
 LINEAR_SHAPES = [(1, 64, 192), (2, 96, 320), (7, 320, 96), (16, 64, 1000), (9, 4104, 200), (12, 1096, 8200), (5, 520, 16400),
-                 (17, 96, 50257 // 16), (64, 4096, 528), (65, 256, 257), (130, 96, 300), (300, 1600, 520),
+                 (17, 96, 50257 // 16), (24, 200, 8200), (21, 1096, 16400), (25, 96, 300), (64, 4096, 528), (65, 256, 257), (130, 96, 300), (300, 1600, 520),
                  (257, 64, 50257 // 8), (520, 72, 33000)]
 
 
