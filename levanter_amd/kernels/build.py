@@ -76,14 +76,17 @@ def find_hipcc() -> Optional[str]:
     return None
 
 
-def source_hash() -> str:
+def source_hash(unit: str = "core") -> str:
+    """Hash of what a unit is built from: the flags, its own sources and defines, and every header."""
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for name in sorted(os.listdir(CSRC)):
-        if name.endswith((".hip", ".h")):
-            h.update(name.encode())
-            with open(os.path.join(CSRC, name), "rb") as f:
-                h.update(f.read())
+    names = sorted({src for src, _, _ in UNITS[unit]} | {n for n in os.listdir(CSRC) if n.endswith(".h")})
+    for name in names:
+        h.update(name.encode())
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(f.read())
+    for _, defines, obj in UNITS[unit]:
+        h.update((" ".join(defines) + obj).encode())
     return h.hexdigest()[:16]
 
 
@@ -119,7 +122,7 @@ def is_current(unit: str = "core") -> bool:
     lib = library_path(unit)
     try:
         with open(_stamp_path(lib)) as f:
-            return os.path.isfile(lib) and f.read().strip() == source_hash()
+            return os.path.isfile(lib) and f.read().strip() == source_hash(unit)
     except OSError:
         return False
 
@@ -160,7 +163,6 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(compile_one, items))
-    digest = source_hash()
     for u in todo:
         lib = paths[u]
         objs = [os.path.join(obj_dir, obj_name) for _, _, obj_name in UNITS[u]]
@@ -170,7 +172,7 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
             raise RuntimeError(f"hipcc failed to link {lib_name(u)}:\n{_filter(r.stderr)}")
         os.replace(tmp, lib)
         with open(_stamp_path(lib), "w") as f:
-            f.write(digest)
+            f.write(source_hash(u))
     _log(f"built {', '.join(lib_name(u) for u in todo)} in {library_dir()} in {time.time() - t0:.0f}s")
     return paths
 
