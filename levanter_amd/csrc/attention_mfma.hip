@@ -342,27 +342,31 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
 
 // ------------------------------------------------------------------------------------------------
 // Decode: one wave per (token, kv head, split). Columns of Q^T are the G = H / KVH query heads that
-// share the kv head. With more than one split the partial results go to the workspace
-//   ws_m, ws_l [token][head][split], ws_o [token][head][split][HD]
-// and a second kernel merges them in the order of the splits. (Merging in the last wave to finish, behind an
-// atomic ticket, was measured: the device-scope fences it needs cost several times the second launch.)
+// share the kv head. With more than one split the partial results are merged in the order of the splits:
+//   wg_merge: the splits of a (token, kv head) are the waves of ONE workgroup (up to DECODE_WG_WAVES); they leave
+//     m, l and o in LDS and, behind a barrier, the workgroup's threads merge them and write the output;
+//   else (more splits than that, or too many query heads per kv head for the LDS): one workgroup per split,
+//     partial results in the workspace  ws_m, ws_l [token][head][split], ws_o [token][head][split][HD],  and a
+//     second kernel merges them. (Merging in the last workgroup to finish, behind an atomic ticket, was measured:
+//     the device-scope fences it needs cost several times the second launch.)
 //
 // k_new != null: the step's new key and value of each token are not in the cache yet. The wave whose key
 // range holds the token's own position takes them from k_new / v_new (rows of the projection's output),
 // uses them in place of what the cache holds there, and writes them to dest[t] = page * PS + offset.
-__global__ void __launch_bounds__(64)
+#define DECODE_WG_WAVES 8
+__global__ void __launch_bounds__(64 * DECODE_WG_WAVES)
 LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
                          bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
                          const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
                          const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
                          const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
                          float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
-                         int H, int KVH, int ps_shift, int splits, float scale, int window) {
+                         int H, int KVH, int ps_shift, int splits, float scale, int window, int wg_merge) {
   const int PS = 1 << ps_shift, ps_mask = PS - 1;
   const float scale_log2 = scale * 1.4426950408889634f;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
   const int fr = lane & 15, g = lane >> 4;
-  const int idx = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+  const int idx = blockIdx.x, kvh = blockIdx.y, z = wg_merge ? (int)(threadIdx.x >> 6) : (int)blockIdx.z;
   const int t = decode_tokens[idx];
   const int G = H / KVH;
   const int pos = positions[t];
@@ -482,6 +486,38 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
     }
     return;
   }
+  if (wg_merge) {
+    // partial results of this wave into LDS [split][query head of the group]: m, l, o[HD]
+    extern __shared__ float merge_s[];
+    float* ms = merge_s;
+    float* ls = ms + splits * G;
+    float* os = ls + splits * G;
+    if (fr < G) {
+      if (g == 0) {
+        ms[z * G + fr] = m;
+        ls[z * G + fr] = l;
+      }
+      float* wo = os + (size_t)(z * G + fr) * HD;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(wo + 16 * dt + 4 * g) = o[dt];
+    }
+    __syncthreads();
+    bf16_t* orow = out + (size_t)t * o_stride + (size_t)kvh * G * HD;
+    for (int e = threadIdx.x; e < G * HD; e += blockDim.x) {
+      const int hq = e / HD, d = e - hq * HD;
+      float mx = -INFINITY;
+      for (int zz = 0; zz < splits; ++zz) mx = fmaxf(mx, ms[zz * G + hq]);
+      float lsum = 0.f, acc = 0.f;
+      for (int zz = 0; zz < splits; ++zz) {  // the maxima are in the base-2 domain
+        const float mz = ms[zz * G + hq];
+        const float wz = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);
+        lsum += ls[zz * G + hq] * wz;
+        acc += os[(size_t)(zz * G + hq) * HD + d] * wz;
+      }
+      orow[(size_t)hq * HD + d] = float_to_bf16(acc / lsum);
+    }
+    return;
+  }
   if (q_pos >= 0) {
     const size_t slot = ((size_t)idx * H + head) * splits + z;
     if (g == 0) {
@@ -552,13 +588,16 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     float* ws_m = (float*)workspace;
     float* ws_l = ws_m + rows;
     float* ws_o = ws_l + rows;
-    dim3 grid(n_decode, KVH, splits);
-    LEV_NAME(attn_decode_hd)<<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages,
-                                                      (bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-                                                      decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest,
-                                                      ws_m, ws_l, ws_o, H, KVH, ps_shift, splits, scale, window);
+    const int G = H / KVH;
+    const size_t merge_bytes = (size_t)splits * G * (HD + 2) * sizeof(float);
+    const int wg_merge = splits > 1 && splits <= DECODE_WG_WAVES && merge_bytes <= 48 * 1024;
+    dim3 grid(n_decode, KVH, wg_merge ? 1 : splits);
+    LEV_NAME(attn_decode_hd)<<<grid, wg_merge ? 64 * splits : 64, wg_merge ? merge_bytes : 0, stream>>>(
+        (const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, positions, token_seq, block_tables,
+        bt_stride, decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest, ws_m, ws_l, ws_o, H, KVH, ps_shift,
+        splits, scale, window, wg_merge);
     if (int rc = lev_check_launch("attention decode")) return rc;
-    if (splits > 1) {
+    if (splits > 1 && !wg_merge) {
       dim3 cgrid(n_decode, H);
       LEV_NAME(attn_combine_hd)<<<cgrid, 64, 0, stream>>>((bf16_t*)out, o_stride, decode_tokens, ws_m, ws_l, ws_o, H, splits);
       if (int rc = lev_check_launch("attention combine")) return rc;

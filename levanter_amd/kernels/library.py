@@ -254,7 +254,10 @@ class HipKernels:
             return 1
         want = max(1, 2048 // max(1, meta.n_decode * n_kv_heads))
         most = max(1, (meta.max_kv_len + 63) // 64)  # at least 64 keys per split
-        return int(min(want, most, 64))
+        splits = int(min(want, most, 64))
+        if splits > 8 and most <= 32:
+            splits = 8  # up to 8 splits are merged inside one workgroup (no second kernel); worth 4 blocks of keys per wave
+        return splits
 
     @staticmethod
     def mfma_attention_supports(head_dim: int, group: int) -> bool:
