@@ -42,14 +42,14 @@ def read_step(out, step, vocab):
     return torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_all_cuttings(name, dtype):
     raw, seed = TINY[name]
     store = torch.float32 if dtype == "float32" else torch.bfloat16
     d = write_model(raw, seed, store)
     weights = read_weights(d)
-    lengths = [70, 45, 100, 37, 64, 33] if name == "A" else [90, 130, 41, 200, 64, 17]
+    lengths = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [130, 66, 35, 97, 64, 18]}[name]
     reqs = TR.random_requests(raw["vocab_size"], lengths, seed + 10)
     rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
     plain = {rid: P.plain_logits(weights, raw, torch.tensor(t), rounding=rounding) for rid, t in reqs.items()}

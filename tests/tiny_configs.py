@@ -1,4 +1,5 @@
-"""The two tiny GPT-2 configurations that the tests use. They differ in every size and option."""
+"""The tiny GPT-2 configurations that the tests use. A and B differ in every size and option; C has sizes that are
+no power of two anywhere (a head size of 112, two heads, an inner width of 100, a vocabulary of 257)."""
 
 TINY_A = {
     "model_type": "gpt2",
@@ -32,4 +33,20 @@ TINY_B = {
     "tie_word_embeddings": True,
 }
 
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1)}
+TINY_C = {
+    "model_type": "gpt2",
+    "n_layer": 2,
+    "n_embd": 224,
+    "n_head": 2,
+    "n_inner": 100,
+    "vocab_size": 257,
+    "n_positions": 130,
+    "layer_norm_epsilon": 1e-3,
+    "activation_function": "silu",
+    "scale_attn_by_inverse_layer_idx": True,
+    "reorder_and_upcast_attn": False,
+    "initializer_range": 0.02,
+    "tie_word_embeddings": True,
+}
+
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
