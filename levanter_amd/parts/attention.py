@@ -49,6 +49,7 @@ class CausalSelfAttention(Mixer):
         self.rotary = None
         if rotary is not None:
             self.rotary = POSITION_ENCODINGS.get(rotary.kind)(rotary, {k: tensors[k] for k in rotary.tensors}, env)
+            self.graph_safe = bool(self.rotary.graph_safe)  # the rotation runs inside this mixer's forward
 
     def cache_requirement(self):
         return PagedKv(self.n_kv_heads, self.head_dim, self.window)

@@ -88,6 +88,12 @@ class StepContext:
 class Part:
     kind: str = ""
 
+    graph_safe = False
+    """True if the part only launches work whose shape is fixed by the step's sizes and reads everything that
+    changes from step to step (tokens, positions, tables) from device memory: such work can be recorded once into
+    a HIP graph and replayed. A part that steers from the host (``ctx.host``, data-dependent shapes, copies to the
+    CPU) leaves it False, and a model with such a part runs every step eagerly. Blocks answer for their members."""
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         self.spec = spec
         self.env = env
@@ -123,10 +129,6 @@ class Mixer(Part):
     ``forward(h, x, ctx, unit, writes_cache)``: adds the mixer's output for ``h`` (compute dtype
     ``[T, dim]``) to the residual ``x`` (float32 ``[T, dim]``) in place; reads (and, if
     ``writes_cache``, first writes) ``unit``."""
-
-    graph_safe = False
-    """True if ``forward`` only launches work whose shape is fixed by the step's sizes and reads everything
-    else from device tensors (no host-side steering by ``ctx.host``): such steps may be captured into a HIP graph."""
 
     def cache_requirement(self):
         return None

@@ -13,6 +13,10 @@ class PreNormBlock(Block):
     def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, feed_forward: FeedForward):
         self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.norm1, self.mixer, self.norm2, self.feed_forward))
+
     def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
         self.mixer.forward(self.norm1(x, ctx), x, ctx, unit, writes_cache)
         self.feed_forward.forward(self.norm2(x, ctx), x, ctx)

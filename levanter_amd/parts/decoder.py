@@ -87,7 +87,11 @@ class DecoderLm:
 
     @property
     def graph_safe(self) -> bool:
-        return all(b.mixer.graph_safe for b in self.blocks)
+        """Every part agrees to be replayed from a HIP graph (a block answers for its members)."""
+        parts = [*self.blocks, self.final_norm, self.head]
+        if self.embedding.position is not None:
+            parts.append(self.embedding.position)
+        return all(getattr(p, "graph_safe", False) for p in parts)
 
     @property
     def max_positions(self) -> Optional[int]:

@@ -15,6 +15,8 @@ from .spec import PartSpec
 
 @FEED_FORWARDS.register("dense_mlp")
 class DenseMlp(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
         p = spec.params

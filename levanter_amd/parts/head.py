@@ -14,6 +14,8 @@ from .spec import PartSpec
 
 @HEADS.register("tied_head")
 class TiedHead(Head):
+    graph_safe = True
+
     """Uses the embedding's table (set by the decoder with ``tie``); holds no second copy."""
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
@@ -31,6 +33,8 @@ class TiedHead(Head):
 
 @HEADS.register("linear_head")
 class LinearHead(Head):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
         self.proj = Linear(tensors["weight"], tensors.get("bias"), spec.params.get("weight_layout", "out_in"), env)

@@ -14,6 +14,8 @@ from .spec import PartSpec
 
 @NORMS.register("layernorm")
 class LayerNorm(Norm):
+    graph_safe = True
+
     rms = False
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):

@@ -13,6 +13,8 @@ from .spec import PartSpec
 
 @POSITION_ENCODINGS.register("learned_absolute")
 class LearnedAbsolutePosition(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
         self.max_positions = int(spec.params["n_positions"])
@@ -24,5 +26,7 @@ class LearnedAbsolutePosition(PositionEncoding):
 
 @POSITION_ENCODINGS.register("none")
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)

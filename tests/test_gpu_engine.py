@@ -498,3 +498,148 @@ def test_graphed_decode_batches_are_filled_up_with_ghost_tokens(dtype):
     for (r, _), h in zip(runners, handles):
         last.append(r.step([StepEntry(h[k], toks[k][h[k].length:h[k].length + 3], [2]) for k in live]).cpu())
     torch.testing.assert_close(last[0], last[1], **tol)
+
+
+def test_a_toy_rotary_position_encoding_registers_and_only_distances_count():
+    """Another position encoding, defined here: queries and keys are rotated by their absolute position before
+    the cache write (pairs (i, i + head_dim/2) of a head), the embedding adds no position. Compared with a plain
+    whole-sequence computation; and a shift of all positions changes nothing, because only distances count."""
+    from levanter_amd.parts import POSITION_ENCODINGS, PartSpec, PositionEncoding
+
+    H, HD, BASE = 4, 16, 100.0
+
+    def angles(pos):  # [T, HD/2]
+        inv = BASE ** (-torch.arange(HD // 2, dtype=torch.float64) / (HD // 2))
+        return pos.double()[:, None] * inv[None, :]
+
+    def plain_rotate(x, pos):  # x [T, H, HD]
+        a = angles(pos)
+        c, s_ = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+        x1, x2 = x[..., : HD // 2], x[..., HD // 2:]
+        return torch.cat([x1 * c - x2 * s_, x2 * c + x1 * s_], -1)
+
+    @POSITION_ENCODINGS.register("toy_rotary")
+    class ToyRotary(PositionEncoding):
+        graph_safe = True  # positions are read from device memory, shapes follow the step's sizes
+
+        def rotate(self, q, k, ctx):
+            pos = ctx.attention.positions.to(torch.float32)
+            inv = BASE ** (-torch.arange(HD // 2, dtype=torch.float32, device=q.device) / (HD // 2))
+            ang = pos[:, None] * inv[None, :]
+            c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            for t in (q, k):  # strided views into the fused projection's output: rotated in place, in 32-bit
+                v = t.view(t.shape[0], -1, HD) if t.is_contiguous() else t.unflatten(1, (-1, HD))
+                x1, x2 = v[..., : HD // 2].float().clone(), v[..., HD // 2:].float().clone()  # copies: float() of float32 is a view
+                v[..., : HD // 2] = (x1 * c - x2 * s_).to(t.dtype)
+                v[..., HD // 2:] = (x2 * c + x1 * s_).to(t.dtype)
+
+    try:
+        d = write_model(TINY_A, 0, torch.float32)
+        w = read_weights(d)
+        t32 = {k: v.float() for k, v in w.items()}
+        spec = _toy_spec()
+        spec.embedding.params["position"] = None  # no learned positions
+        spec.max_positions = None
+        for layer in spec.layers:
+            layer.mixer.params["rotary"] = PartSpec("toy_rotary", {}, {})
+        toks = torch.randint(0, 512, (60,), generator=torch.Generator().manual_seed(8)).tolist()
+
+        def plain(first_pos):
+            pos = torch.arange(first_pos, first_pos + 60)
+            x = w["wte.weight"][torch.tensor(toks)]
+            for i in range(2):
+                p = f"h.{i}."
+                hh = P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5)
+                q, k, v = P.plain_split_qkv(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"]), H)  # [H, T, HD]
+                q = plain_rotate(q.transpose(0, 1), pos).transpose(0, 1)
+                k = plain_rotate(k.transpose(0, 1), pos).transpose(0, 1)
+                o = P.plain_causal_attention(q, k, v)
+                x = x + P.plain_linear(o.transpose(0, 1).reshape(60, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+                x = x + P.plain_mlp(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5), w, p, TINY_A)
+            return P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+
+        want = plain(0)
+        torch.testing.assert_close(plain(37), want, rtol=1e-9, atol=1e-9)  # the plain statement itself: only distances count
+        for cuts in ([60], [23, 2, 30, 1, 1, 1, 1, 1]):
+            got, _, _ = _run_cut(spec, t32, "float32", toks, cuts)
+            torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=2e-5)
+    finally:
+        POSITION_ENCODINGS.unregister("toy_rotary")
+
+
+def test_a_toy_feed_forward_with_routing_registers_builds_and_steps():
+    """A feed-forward with routing, defined here: a router picks one of two experts per token (the larger of two
+    32-bit router logits), each expert is a dense unit run by the framework's own GEMM on the rows sent to it.
+    It steers from the host (row lists of changing length), so it is not graph-safe and the model steps eagerly."""
+    from levanter_amd.parts import FEED_FORWARDS, FeedForward, PartSpec, TensorSpec
+    from levanter_amd.parts.linear import Linear
+
+    D, F = 64, 256
+
+    @FEED_FORWARDS.register("toy_top1_experts")
+    class Top1Experts(FeedForward):
+        def __init__(self, spec, tensors, env):
+            super().__init__(spec, tensors, env)
+            self.router = tensors["router"].to(env.device, torch.float32)  # [2, D]
+            self.ups = [Linear(tensors[f"up{e}.weight"], tensors[f"up{e}.bias"], "in_out", env) for e in range(2)]
+            self.downs = [Linear(tensors[f"down{e}.weight"], tensors[f"down{e}.bias"], "in_out", env) for e in range(2)]
+
+        def forward(self, h, x, ctx):
+            choice = (h.float() @ self.router.T).argmax(-1)  # router logits in 32-bit
+            for e in range(2):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                m = self.ups[e](h[rows].contiguous(), ctx, activation="gelu_new")
+                y = torch.zeros(rows.numel(), D, dtype=torch.float32, device=h.device)
+                self.downs[e](m, ctx, residual=y)
+                x[rows] += y
+
+    try:
+        d = write_model(TINY_A, 0, torch.float32)
+        w = read_weights(d)
+        t32 = {k: v.float() for k, v in w.items()}
+        g = torch.Generator().manual_seed(12)
+        extra = {"h.1.moe.router": torch.randn(2, D, generator=g)}
+        for e in range(2):  # expert 0 is layer 1's own dense unit, expert 1 a second one
+            src = "h.1.mlp." if e == 0 else None
+            extra[f"h.1.moe.up{e}.weight"] = t32["h.1.mlp.c_fc.weight"] if src else torch.randn(D, F, generator=g) * 0.05
+            extra[f"h.1.moe.up{e}.bias"] = t32["h.1.mlp.c_fc.bias"] if src else torch.randn(F, generator=g) * 0.05
+            extra[f"h.1.moe.down{e}.weight"] = t32["h.1.mlp.c_proj.weight"] if src else torch.randn(F, D, generator=g) * 0.05
+            extra[f"h.1.moe.down{e}.bias"] = t32["h.1.mlp.c_proj.bias"] if src else torch.randn(D, generator=g) * 0.05
+        tensors = dict(t32, **extra)
+        spec = _toy_spec()
+        names = ["router"] + [f"{n}{e}.{k}" for e in range(2) for n in ("up", "down") for k in ("weight", "bias")]
+        spec.layers[1].feed_forward = PartSpec("toy_top1_experts", {},
+                                               {n: TensorSpec("h.1.moe." + n, tuple(tensors["h.1.moe." + n].shape)) for n in names})
+        toks = torch.randint(0, 512, (48,), generator=torch.Generator().manual_seed(13)).tolist()
+        wd = {k: v.double() for k, v in tensors.items()}
+        x = P.plain_embed(torch.tensor(toks), torch.arange(48), w["wte.weight"], w["wpe.weight"])
+        x = P.plain_block(x, w, TINY_A, 0)
+        p = "h.1."
+        hh = P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5)
+        q, k, v = P.plain_split_qkv(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"]), 4)
+        o = P.plain_causal_attention(q, k, v)
+        x = x + P.plain_linear(o.transpose(0, 1).reshape(48, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+        h2 = P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5)
+        logits_r = h2 @ wd["h.1.moe.router"].T
+        choice = logits_r.argmax(-1)
+        assert 5 < int(choice.sum()) < 43  # both experts get tokens
+        assert float((logits_r[:, 0] - logits_r[:, 1]).abs().min()) > 1e-3  # no token on the fence between them
+        act = P.plain_activation("gelu_new")
+        y = torch.zeros_like(x)
+        for e in range(2):
+            rows = choice == e
+            m = act(h2[rows] @ wd[f"h.1.moe.up{e}.weight"] + wd[f"h.1.moe.up{e}.bias"])
+            y[rows] = m @ wd[f"h.1.moe.down{e}.weight"] + wd[f"h.1.moe.down{e}.bias"]
+        x = x + y
+        want = P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+        for cuts in ([48], [17, 2, 28, 1]):
+            got, _, _ = _run_cut(spec, tensors, "float32", toks, cuts)
+            torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=2e-5)
+        from levanter_amd.parts import DecoderLm
+
+        assert not DecoderLm(spec, tensors, _env("float32")).graph_safe
+        assert DecoderLm(_toy_spec(), t32, _env("float32")).graph_safe
+    finally:
+        FEED_FORWARDS.unregister("toy_top1_experts")
