@@ -8,7 +8,5 @@ extern "C" long lev_attention_mfma_workspace(int n_decode, int splits, int H, in
   return (long)n_decode * splits * H * (HD + 2) * (long)sizeof(float);
 }
 
-extern "C" int lev_attention_mfma_max_head_dim() { return 128; }
-
 // query rows of one prefill tile: the host cuts runs longer than one token into tiles of at most this many rows
 extern "C" int lev_attention_prefill_tile_rows() { return PF_ROWS; }
