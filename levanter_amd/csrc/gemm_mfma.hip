@@ -598,12 +598,34 @@ splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict_
   }
 }
 
+// Into how many k ranges the stream kernel splits K. Three things are weighed against each other, each relative to
+// the time of streaming the weights once:
+//   balance: the workgroups (column tiles x ranges) go over 256 CUs in rounds, and the last round should be full.
+//     With 192 column tiles 3 ranges give 576 workgroups: a quarter of the CUs takes three, the rest two, and the
+//     kernel lasts as long as with 2 ranges; 4 ranges give three to every CU;
+//   latency: with fewer than two workgroups per CU the loads in flight do not cover the memory latency;
+//   the partial sums: every range writes M x N floats that the second kernel reads again (4 S M / K of the weights'
+//     bytes, but mostly out of the caches: weighted half), and the second launch itself.
+static int stream_splits(int M, int N, int K) {
+  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+  const int s_max = chunks / 2 < 16 ? (chunks / 2 < 1 ? 1 : chunks / 2) : 16;  // at least two chunks each
+  int best = 1;
+  double best_cost = 1e30;
+  for (int s = 1; s <= s_max; ++s) {
+    const long wgs = (long)tiles * s;
+    const double imbalance = ((double)((wgs + 255) / 256) / s) / (tiles / 256.0);
+    const double cost = imbalance * (wgs < 512 ? 1.5 : 1.0) + (s > 1 ? 0.1 + 2.0 * s * M / K : 0.0);
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
   if (M <= SKINNY_MAX_M || M > 128) return 0;
-  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
-  int S = (512 + tiles - 1) / tiles;
-  if (S > chunks / 2) S = chunks / 2;
-  if (S < 1) S = 1;
+  const int S = stream_splits(M, N, K);
   return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
 }
 
@@ -611,10 +633,8 @@ template <typename TO>
 static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
                          long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
   if ((size_t)M * lda >= (1ull << 32)) return lev_fail("linear: the activation matrix is too large (M=%d lda=%ld)", M, lda);
-  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
-  int S = (512 + tiles - 1) / tiles;  // enough workgroups for two per CU
-  if (S > chunks / 2) S = chunks / 2;   // at least two chunks each
-  if (S < 1) S = 1;
+  const int tiles = (N + 63) / 64;
+  const int S = stream_splits(M, N, K);
   if (S > 1 && !workspace) return lev_fail("linear: M=%d N=%d K=%d needs a workspace of lev_linear_mfma_workspace bytes", M, N, K);
   dim3 grid(tiles, S);
   if (M <= 32)
