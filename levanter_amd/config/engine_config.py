@@ -46,6 +46,8 @@ class InferenceEngineConfig:
     """Return the log-probability of every generated token (engine.py:102)."""
     max_state_slots: Optional[int] = None
     """Slots of fixed-size per-request state; None: max_seqs. (Ours.)"""
+    decode_lookahead: bool = True
+    """Launch the next step of single tokens before the tokens of the running one are read back. (Ours.)"""
 
     def __post_init__(self):
         if self.page_size <= 0 or self.page_size % 16 != 0:

@@ -27,6 +27,14 @@ logger = logging.getLogger(__name__)
 __all__ = ["InferenceEngine", "Request", "SeqDecodingParams", "GenerationResult", "InferenceEngineConfig"]
 
 
+class _Launched:
+    """A step that runs on the GPU: its plan, its sampling under way, and whether its sampled tokens can feed the
+    next step on the device (every entry one decoded token that wants logits)."""
+
+    def __init__(self, plan, sample, feeds: bool):
+        self.plan, self.sample, self.feeds = plan, sample, feeds
+
+
 class InferenceEngine:
     def __init__(self, model, config: InferenceEngineConfig, env: BuildEnv, allocate: bool = True):
         self.model = model
@@ -37,6 +45,7 @@ class InferenceEngine:
         self.sampler = Sampler(env.kernels, env.device)
         self.scheduler = Scheduler(self.cache, config, self.runner.max_len)
         self.stats = {"steps": 0, "tokens_in": 0, "device_s": 0.0}
+        self._pending: Optional[_Launched] = None  # a step launched ahead of the one being committed
 
     # ---- construction -------------------------------------------------------------------------
     @classmethod
@@ -100,25 +109,58 @@ class InferenceEngine:
 
     # ---- one scheduler iteration -----------------------------------------------------------------------
     def step(self) -> List[Sequence_]:
-        """Plan a step, run it, sample, commit. Returns the sequences that finished in it."""
-        plan: List[PlannedEntry] = self.scheduler.plan()
-        if not plan:
-            return []
+        """Commit one step: plan it and run it (unless it was launched ahead already), sample, append the tokens.
+        Returns the sequences that finished in it.
+
+        Decoding is pipelined: while the GPU runs a step of single tokens, the step after it is planned and launched
+        with its token ids taken from the sampler's output on the device, and only then are the first step's tokens
+        read back. The GPU never waits for the host between two decode steps. What cannot be known without the tokens
+        (a stop sequence that ends a request) is settled afterwards: the request's row of the step launched ahead is
+        ignored, and what that row wrote lies in pages that its request no longer owns and nobody reads."""
+        pend = self._pending
+        self._pending = None
+        if pend is None:
+            plan: List[PlannedEntry] = self.scheduler.plan()
+            if not plan:
+                return []
+            pend = self._launch(plan, None)
+        nxt = None
+        if self.config.decode_lookahead and pend.feeds:
+            ahead = self.scheduler.plan_lookahead(pend.plan)
+            if ahead is not None:
+                nxt = self._launch(ahead[0], (pend.sample.tokens, ahead[1]))
+        toks, lps = ([], []) if pend.sample is None else self.sampler.read(pend.sample)
+        finished = self.scheduler.commit(pend.plan, toks, lps)
+        if nxt is not None:
+            if all(e.seq.done for e in nxt.plan):  # every request of the step launched ahead has ended meanwhile
+                self.sampler.read(nxt.sample)
+            else:
+                self._pending = nxt
+        return finished
+
+    def _launch(self, plan: List[PlannedEntry], feed) -> "_Launched":
+        """Run a planned step and start sampling; nothing is waited for. ``feed = (device tokens, rows)``: the
+        entries' tokens are the sampled tokens of the step before, still on the device."""
         entries = [StepEntry(e.seq.handle, e.tokens, [len(e.tokens) - 1] if e.wants_logits else []) for e in plan]
         t0 = time.perf_counter()
-        logits = self.runner.step(entries, copy_out=False)
+        token_feed = None
+        if feed is not None:
+            device_tokens, rows = feed
+            same = rows == list(range(len(rows))) and len(rows) == int(device_tokens.numel())
+            token_feed = (device_tokens, None if same else torch.tensor(rows, dtype=torch.int64, device=device_tokens.device), len(rows))
+        logits = self.runner.step(entries, copy_out=False, token_feed=token_feed)
         wanted = [e for e in plan if e.wants_logits]
-        toks: List[int] = []
-        lps: List[float] = []
+        sample = None
         if wanted:
             temps = [e.seq.request.decode_params.temperature for e in wanted]
             keys = [e.seq.key for e in wanted]
             positions = [e.seq.n_cached - 1 for e in wanted]  # position of the token whose logits are sampled
-            toks, lps = self.sampler.to_host(logits, temps, keys, positions)
+            sample = self.sampler.launch(logits, temps, keys, positions)
         self.stats["steps"] += 1
         self.stats["tokens_in"] += sum(len(e.tokens) for e in plan)
         self.stats["device_s"] += time.perf_counter() - t0
-        return self.scheduler.commit(plan, toks, lps)
+        feeds = bool(plan) and all(e.wants_logits and len(e.tokens) == 1 for e in plan)
+        return _Launched(plan, sample, feeds)
 
     def generate(self, requests: Sequence[Request]) -> GenerationResult:
         seqs = self.enqueue_requests(requests)
@@ -140,5 +182,8 @@ class InferenceEngine:
 
     def reset(self) -> None:
         """Drop every request and give back all pages and slots (engine.py:761-776)."""
+        if self._pending is not None and self._pending.sample is not None:
+            self.sampler.read(self._pending.sample)  # let the step launched ahead finish before its pages go
+        self._pending = None
         self.scheduler.abort_all()
         self.cache.reset()

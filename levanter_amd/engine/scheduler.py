@@ -186,6 +186,35 @@ class Scheduler:
             n_prefill += 1
         return entries, starved
 
+    def plan_lookahead(self, pending: List[PlannedEntry]) -> Optional[Tuple[List[PlannedEntry], List[int]]]:
+        """The step after ``pending`` (a launched step whose sampled tokens are not on the host yet), if it can be
+        decided without them: ``pending`` is every running request decoding one token, nobody waits for admission,
+        and the pools hold the pages. Requests that end by length with ``pending``'s token are left out; one that
+        ends by a stop sequence cannot be foreseen and is skipped when this step is committed. Returns the entries
+        (their token lists hold a placeholder) and, for each, its row among ``pending``'s entries; None: plan as usual."""
+        if self.waiting or not pending or len(pending) != len(self.running) or len(pending) > self.cfg.imputed_max_tokens_per_round:
+            return None
+        if any(not e.wants_logits or len(e.tokens) != 1 or e.seq.done for e in pending):
+            return None
+        free = [g.pool.n_free for g in self.cache.groups]
+        entries: List[PlannedEntry] = []
+        rows: List[int] = []
+        for i, e in enumerate(pending):
+            seq = e.seq
+            if len(seq.tokens) + 1 >= min(seq.request.decode_params.max_num_tokens, self.max_len):
+                continue  # pending's token is its last
+            need = [g.blocks_needed(seq.handle.slot, seq.handle.length, seq.handle.length + 1) for g in self.cache.groups]
+            if any(nd > fr for nd, fr in zip(need, free)):
+                return None  # pages run out: the ordinary plan decides whom to preempt
+            for k, nd in enumerate(need):
+                free[k] -= nd
+            entries.append(PlannedEntry(seq, [0], True))
+            rows.append(i)
+        if not entries:
+            return None
+        self._steps_since_admission += 1
+        return entries, rows
+
     def _preempt(self, seq: Sequence_) -> None:
         """Free the sequence's pages and slot; it re-enters at the head of the queue and recomputes
         the cache of all its tokens so far. Its generated tokens and sampling key are kept."""
@@ -207,6 +236,8 @@ class Scheduler:
                 continue
             seq, tok, lp = e.seq, int(sampled[i]), float(logprobs[i])
             i += 1
+            if seq.done:  # it ended by a stop sequence after this step had been launched ahead
+                continue
             seq.tokens.append(tok)
             seq.generated.append(tok)
             seq.logprobs.append(lp)

@@ -88,10 +88,13 @@ class ModelRunner:
                     raise StepError(f"request {rid!r}: wanted place {w} is not among its {n} tokens")
 
     # ------------------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], copy_out: bool = True) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], copy_out: bool = True, token_feed=None) -> torch.Tensor:
         """Run the entries as one batch. Returns float32 logits [wanted, vocab] in the order of the
         entries and of their ``want``. Raises ``OutOfPages`` (nothing changed) if a pool is too small.
-        ``copy_out=False`` may return a buffer that the next step overwrites (the sampler reads it at once)."""
+        ``copy_out=False`` may return a buffer that the next step overwrites (the sampler reads it at once).
+        ``token_feed = (device_tokens int32 [R], rows, n)``: the n entries are single tokens that are not known on the
+        host yet; entry i's token is ``device_tokens[rows[i]]`` (``rows`` None: ``device_tokens[i]``), the sampler's
+        output of the step before, put in place on the device after the step's tables have been uploaded."""
         entries = list(entries)
         self._validate(entries)
         if not entries:
@@ -104,12 +107,16 @@ class ModelRunner:
             self.cache.extend(e.handle, len(e.tokens))
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
         batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
+        if token_feed is not None and any(len(e.tokens) != 1 for e in entries):
+            raise StepError("tokens can be fed from the device to entries of a single token only")
         if graphable:
-            logits = self._run_graphed(batch)[:batch.n_rows_real]
+            logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
             if copy_out:
                 logits = logits.clone()
         else:
-            logits = self.model.forward(self._make_ctx(self._upload(batch.host), batch, self._workspaces), batch.rows_view)
+            dev = self._upload(batch.host)
+            self._feed_tokens(dev, batch, token_feed)
+            logits = self.model.forward(self._make_ctx(dev, batch, self._workspaces), batch.rows_view)
         for e in entries:
             self.cache.advance(e.handle, len(e.tokens))
         return logits
@@ -222,7 +229,19 @@ class ModelRunner:
         return t.pin_memory().to(self.env.device, non_blocking=True)
 
     # ---- decode steps as HIP graphs --------------------------------------------------------
-    def _run_graphed(self, b: "HostBatch") -> torch.Tensor:
+    @staticmethod
+    def _feed_tokens(dev: torch.Tensor, b: "HostBatch", token_feed) -> None:
+        """Entry i's token id comes from ``device_tokens[rows[i]]`` (the entries are the first tokens of the step)."""
+        if token_feed is None:
+            return
+        device_tokens, rows, n = token_feed
+        dst = dev[b.offs[0]:b.offs[0] + n]
+        if rows is None:  # the same requests in the same order as in the step before
+            dst.copy_(device_tokens[:n])
+        else:
+            torch.index_select(device_tokens, 0, rows, out=dst)
+
+    def _run_graphed(self, b: "HostBatch", token_feed=None) -> torch.Tensor:
         """A step of single tokens has a kernel sequence that depends only on (requests, wanted rows,
         blocks per request): the second time such a step comes it is captured into a HIP graph whose
         inputs live in a fixed device buffer; later steps copy their tables there and replay it."""
@@ -230,7 +249,9 @@ class ModelRunner:
         entry = self._graphs.get(key)
         if entry is None:  # first time: run eagerly (also loads every kernel the graph will need)
             self._graphs[key] = "seen"
-            return self.model.forward(self._make_ctx(self._upload(b.host), b, self._workspaces), b.rows_view)
+            dev = self._upload(b.host)
+            self._feed_tokens(dev, b, token_feed)
+            return self.model.forward(self._make_ctx(dev, b, self._workspaces), b.rows_view)
         if entry == "seen":
             if len(self._graphs) > MAX_GRAPHS:
                 self._graphs = {k: v for k, v in self._graphs.items() if v == "seen"}
@@ -239,6 +260,7 @@ class ModelRunner:
                            pinned=torch.zeros(n, dtype=torch.int32).pin_memory(), copied=torch.cuda.Event())
             entry.pinned.numpy()[:] = b.host
             entry.static.copy_(entry.pinned, non_blocking=True)
+            self._feed_tokens(entry.static, b, token_feed)
             ctx = self._make_ctx(entry.static, b, {})
             torch.cuda.current_stream().synchronize()
             entry.graph = torch.cuda.CUDAGraph()
@@ -249,6 +271,7 @@ class ModelRunner:
             entry.copied.synchronize()  # the previous copy out of the pinned buffer is done
             entry.pinned.numpy()[:] = b.host
             entry.static.copy_(entry.pinned, non_blocking=True)
+            self._feed_tokens(entry.static, b, token_feed)
         entry.copied.record()
         entry.graph.replay()
         return entry.logits

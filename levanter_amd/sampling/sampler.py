@@ -67,7 +67,32 @@ class Sampler:
 
     def to_host(self, logits: torch.Tensor, temperatures, keys, positions) -> Tuple[list, list]:
         """Sample and bring tokens and log-probabilities to the host with one copy (one synchronisation)."""
+        return self.read(self.launch(logits, temperatures, keys, positions))
+
+    def launch(self, logits: torch.Tensor, temperatures, keys, positions) -> "PendingSample":
+        """Sample and start the copy of tokens and log-probabilities to the host without waiting for it. The tokens
+        stay on the device too (``PendingSample.tokens``): the next step may be fed from there."""
         r = logits.shape[0]
-        self(logits, temperatures, keys, positions)
-        host = self._last_out.cpu()
-        return host[:r].tolist(), host[r:].view(torch.float32).tolist()
+        tokens, _ = self(logits, temperatures, keys, positions)
+        out = self._last_out
+        if self.device.type == "cpu":
+            return PendingSample(r, tokens, out.clone(), None)
+        host = torch.empty(2 * r, dtype=torch.int32).pin_memory()
+        host.copy_(out, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return PendingSample(r, tokens, host, done)
+
+    @staticmethod
+    def read(pending: "PendingSample") -> Tuple[list, list]:
+        if pending.done is not None:
+            pending.done.synchronize()
+        r = pending.rows
+        return pending.host[:r].tolist(), pending.host[r:].view(torch.float32).tolist()
+
+
+class PendingSample:
+    """A sampling whose copy to the host is under way."""
+
+    def __init__(self, rows: int, tokens: torch.Tensor, host: torch.Tensor, done):
+        self.rows, self.tokens, self.host, self.done = rows, tokens, host, done

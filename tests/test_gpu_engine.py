@@ -643,3 +643,37 @@ def test_a_toy_feed_forward_with_routing_registers_builds_and_steps():
         assert DecoderLm(_toy_spec(), t32, _env("float32")).graph_safe
     finally:
         FEED_FORWARDS.unregister("toy_top1_experts")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_launched_ahead_give_the_same_generation(dtype):
+    """The engine launches a decode step before the tokens of the step before are on the host (they are fed on the
+    device). With and without that the generations are the same: greedy and sampled requests, a stop sequence that
+    ends a request while a step with it is already under way, requests that end by length at different times."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import InferenceEngine, Request, SeqDecodingParams
+
+    raw, seed = TINY["B"]
+    d = write_model(raw, seed, torch.float32 if dtype == "float32" else torch.bfloat16)
+
+    def run(lookahead):
+        engine = InferenceEngine.from_pretrained(d, InferenceEngineConfig(max_pages=48, max_seqs=6, page_size=16, max_pages_per_seq=8,
+                                                                          compute_dtype=dtype, decode_lookahead=lookahead, seed=5))
+        first = engine.generate([Request(prompt_tokens=[11, 12, 13, 14], request_id=9, max_new_tokens=12)]).tokens[0]
+        stop = [first[5], first[6]]  # a stop sequence that the greedy continuation really produces
+        engine.reset()
+        reqs = [Request(prompt_tokens=[11, 12, 13, 14], request_id=0, decode_params=SeqDecodingParams(max_num_tokens=60, stop_tokens=[stop])),
+                Request(prompt_tokens=[7], request_id=1, max_new_tokens=9),
+                Request(prompt_tokens=list(range(40, 70)), request_id=2, max_new_tokens=20, temperature=0.8),
+                Request(prompt_tokens=[3, 1, 4, 1, 5], request_id=3, max_new_tokens=33, temperature=1.3)]
+        res = engine.generate(reqs)
+        assert engine._pending is None
+        engine.cache.check_invariants()
+        return res.tokens, res.finish_reasons, first
+
+    tok_a, why_a, first = run(True)
+    tok_b, why_b, _ = run(False)
+    assert tok_a == tok_b and why_a == why_b
+    stop = first[5:7]
+    n_stop = next(n for n in range(2, 13) if first[n - 2:n] == stop)  # the greedy continuation up to the stop sequence's first end
+    assert why_a[0] == "stop" and tok_a[0] == first[:n_stop] and [len(t) for t in tok_a[1:]] == [9, 20, 33]

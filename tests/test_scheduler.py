@@ -195,3 +195,31 @@ def test_temperature_sampling_depends_on_request_and_position_only():
     assert len(set(alone)) > 3  # it is sampling, not the argmax
     again = run([Request(prompt_tokens=mine.prompt_tokens, request_id=8, max_new_tokens=12, temperature=5.0)]).tokens[0]
     assert again != alone  # another request id, another key
+
+
+def test_steps_launched_ahead_change_nothing():
+    """Decode steps are launched before the tokens of the step before are read back. The same requests with and
+    without that: the same tokens, reasons and log-probabilities, although a stop sequence ends requests after a
+    step with them has been launched already, requests end by length at different times (the rows of the step
+    launched ahead are then a selection of the rows before), and a request arrives while others decode."""
+    def run(lookahead):
+        engine, model = make_engine(DummyModel(vocab_size=40, count=True), decode_lookahead=lookahead, enable_logprobs=True, max_seqs=8)
+        reqs = [Request(prompt_tokens=[1, 2, 3], request_id=0, decode_params=SeqDecodingParams(max_num_tokens=30, stop_tokens=[[9, 10]]), enable_logprobs=True),
+                Request(prompt_tokens=[20], request_id=1, max_new_tokens=5, enable_logprobs=True),
+                Request(prompt_tokens=[5, 6], request_id=2, max_new_tokens=12, temperature=0.9, enable_logprobs=True),
+                Request(prompt_tokens=[30, 31, 32, 33], request_id=3, decode_params=SeqDecodingParams(max_num_tokens=25, stop_tokens=[[38]]))]
+        seqs = engine.enqueue_requests(reqs[:3])
+        for _ in range(4):
+            engine.step()
+        seqs += engine.enqueue_requests(reqs[3:])  # arrives while a step launched ahead is under way
+        while not all(s.done for s in seqs):
+            engine.step()
+        assert engine._pending is None and all_released(engine)
+        return [(list(s.generated), s.finish_reason, [round(x, 5) for x in s.logprobs]) for s in seqs], model.batches
+
+    with_la, batches_la = run(True)
+    without, batches = run(False)
+    assert with_la == without
+    assert with_la[0][0][-2:] == [9, 10] and with_la[0][1] == "stop" and with_la[1][1] == "length"
+    # a step launched ahead carried one row too many whenever a stop sequence ended a request: more rows in all, never fewer steps
+    assert sum(map(sum, batches_la)) > sum(map(sum, batches)) and len(batches_la) >= len(batches)
