@@ -2,7 +2,7 @@
 //   y = act(a . w^T + bias) (+ residual),  a [M, K] (row stride lda), w [N, K], y [M, N] bf16 or f32.
 // Three kernels, chosen by M:
 //   tile kernel   (M > 128): a 256x256, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
-//                 operands staged through LDS, global loads two k-tiles ahead in registers;
+//                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
 //   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
 //                 straight into MFMA operand registers, K is split over workgroups and a second kernel
 //                 adds the partial sums in a fixed order;
@@ -305,8 +305,8 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns 16 output columns; its WAVES waves split K. A wave takes pairs of
-// adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
+// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns 16 output columns; its WAVES
+// waves split K. A wave takes pairs of adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
 //   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
 //   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
 //            for rows 8..15 of a pair - and turned into the operand layout (row l%16, k-group l/16) through a
