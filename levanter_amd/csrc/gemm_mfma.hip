@@ -1,7 +1,7 @@
 // bfloat16 matrix products on the matrix cores (MFMA), 32-bit accumulation, fused epilogue:
 //   y = act(a . w^T + bias) (+ residual),  a [M, K] (row stride lda), w [N, K], y [M, N] bf16 or f32.
 // Three kernels, chosen by M:
-//   tile kernel   (M > 128): a 256x256, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
+//   tile kernel   (M > 128): a 256x256, 256x192, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
 //   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
 //                 straight into MFMA operand registers, K is split over workgroups and a second kernel
@@ -669,19 +669,25 @@ static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const f
   } else {
     if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
       return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
-    // Estimated time of each tile shape: rounds of workgroups over the 256 CUs (two 128 x 128 workgroups fit
-    // a CU) times the k-tiles plus a fixed cost for a tile's first loads and its epilogue. The constants are
-    // microseconds measured on MI355X; only their ratios matter.
+    // Estimated time of each tile shape: rounds of workgroups over the 256 CUs times (k-tiles x the shape's time per
+    // k-tile + a fixed cost for a tile's first loads and its epilogue). Two 128 x 128 workgroups fit a CU and then
+    // share it; up to 256 of them have a CU each. The constants are microseconds measured on MI355X.
     const long nk = (K + TK - 1) / TK;
-    auto estimate = [&](int bm, int bn, long slots, double us_per_ktile) {
-      const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-      return (double)((tiles + slots - 1) / slots) * (nk * us_per_ktile + 9.0);
+    auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    auto estimate = [&](int bm, int bn, double us_per_ktile, double fixed) {
+      return (double)((tiles(bm, bn) + 255) / 256) * (nk * us_per_ktile + fixed);
     };
-    const double e256 = estimate(256, 256, 256, 2.0), e256x128 = estimate(256, 128, 256, 1.0), e128 = estimate(128, 128, 512, 1.05);
+    const double e[4] = {estimate(256, 256, 1.72, 13.0), estimate(256, 192, 1.36, 11.0), estimate(256, 128, 0.97, 9.0),
+                         tiles(128, 128) <= 256 ? nk * 0.6 + 7.0 : (double)((tiles(128, 128) + 511) / 512) * (nk * 1.05 + 9.0)};
+    int best = 0;
+    for (int i = 1; i < 4; ++i)
+      if (e[i] < e[best]) best = i;
     int rc;
-    if (e256 <= e256x128 && e256 <= e128)
+    if (best == 0)
       rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
-    else if (e256x128 <= e128)
+    else if (best == 1)
+      rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    else if (best == 2)
       rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
     else
       rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
