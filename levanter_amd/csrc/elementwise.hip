@@ -71,11 +71,15 @@ norm_reg_kernel(const float* __restrict__ x, const float* __restrict__ w, const 
   __shared__ float red[NT / 64];
   const int r = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * D;
-  float4 v[NV];
+  // the row, and scale and shift with it: their latency passes during the two reductions
+  float4 v[NV], wv[NV], bv[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int d = (threadIdx.x + i * NT) * 4;
-    v[i] = d < D ? *reinterpret_cast<const float4*>(xr + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool ok = d < D;
+    v[i] = ok ? *reinterpret_cast<const float4*>(xr + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+    wv[i] = ok ? *reinterpret_cast<const float4*>(w + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+    bv[i] = ok && b ? *reinterpret_cast<const float4*>(b + d) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
   float mean = 0.f;
   if (!rms) {
@@ -99,13 +103,9 @@ norm_reg_kernel(const float* __restrict__ x, const float* __restrict__ w, const 
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int d = (threadIdx.x + i * NT) * 4;
-    if (d < D) {
-      const float4 wv = *reinterpret_cast<const float4*>(w + d);
-      float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (b) bv = *reinterpret_cast<const float4*>(b + d);
-      store4<TO>(o + d, (v[i].x - mean) * rstd * wv.x + bv.x, (v[i].y - mean) * rstd * wv.y + bv.y,
-                 (v[i].z - mean) * rstd * wv.z + bv.z, (v[i].w - mean) * rstd * wv.w + bv.w);
-    }
+    if (d < D)
+      store4<TO>(o + d, (v[i].x - mean) * rstd * wv[i].x + bv[i].x, (v[i].y - mean) * rstd * wv[i].y + bv[i].y,
+                 (v[i].z - mean) * rstd * wv[i].z + bv[i].z, (v[i].w - mean) * rstd * wv[i].w + bv[i].w);
   }
 }
 
@@ -139,9 +139,13 @@ __global__ void norm_kernel(const float* __restrict__ x, const float* __restrict
 template <typename TO>
 static void launch_norm(const float* x, const float* w, const float* b, TO* out, const int* rows, int n_rows, int D, float eps,
                         int rms, hipStream_t stream) {
-  if ((D & 3) == 0 && D <= 256 * 4 * 2)
+  // rows in registers as vectors of 4: needs D % 4 == 0 and 16-byte aligned pointers
+  const bool vec = (D & 3) == 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)out) & 15) == 0;
+  if (vec && D <= 256 * 4 * 2)
     norm_reg_kernel<TO, 256, 2><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
-  else if ((D & 3) == 0 && D <= 256 * 4 * 8)
+  else if (vec && D <= 256 * 4 * 4)
+    norm_reg_kernel<TO, 256, 4><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+  else if (vec && D <= 256 * 4 * 8)
     norm_reg_kernel<TO, 256, 8><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
   else
     norm_kernel<TO, 256><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
