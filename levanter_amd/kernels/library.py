@@ -148,8 +148,8 @@ class HipKernels:
         D = x.shape[1]
         n = out.shape[0]
         _req(x.dtype == torch.float32 and x.is_contiguous(), "norm: x must be contiguous float32")
-        _req(weight.dtype == torch.float32 and weight.numel() == D, "norm: weight must be float32 [D]")
-        _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == D), "norm: bias must be float32 [D]")
+        _req(weight.dtype == torch.float32 and weight.numel() == D and weight.is_contiguous(), "norm: weight must be contiguous float32 [D]")
+        _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == D and bias.is_contiguous()), "norm: bias must be contiguous float32 [D]")
         _req(out.is_contiguous() and out.shape[1] == D and out.dtype in _DT, "norm: bad out")
         if rows is None:
             _req(n == x.shape[0], "norm: out must have as many rows as x")

@@ -49,7 +49,8 @@ def test_embed(K, dtype, T, D, V, P):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,D,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (33, 1600, 1e-5), (4, 4100, 1e-3)])
+@pytest.mark.parametrize("T,D,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (33, 1600, 1e-5), (8, 4096, 1e-5), (4, 4100, 1e-3), (3, 6144, 1e-5),
+                                     (2, 8200, 1e-5), (3, 1602, 1e-5)])  # rows held in registers up to 8192 wide, and the general kernel
 @pytest.mark.parametrize("rms", [False, True])
 def test_norm(K, out_dtype, T, D, eps, rms):
     x = _rand(T, D, scale=3.0, seed=4) + 1.5
@@ -69,6 +70,19 @@ def test_norm(K, out_dtype, T, D, eps, rms):
     torch.testing.assert_close(got2.cpu().float(), want2.float(), **tol)
 
 
+def test_norm_of_unaligned_views(K):
+    # a weight vector that starts 4 bytes into its storage cannot be read as vectors of four
+    D = 96
+    x = _rand(3, D, scale=2.0, seed=1)
+    w_store, b_store = _rand(D + 1, seed=2).to(DEV), _rand(D + 1, seed=3).to(DEV)
+    w, b = w_store[1:], b_store[1:]
+    want = torch.empty(3, D)
+    EMU.norm(x, w.cpu(), b.cpu(), 1e-5, want)
+    got = torch.empty(3, D, device=DEV)
+    K.norm(x.to(DEV), w, b, 1e-5, got)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
 def test_norm_constant_row_gives_bias(K):
     x = torch.full((2, 96), 7.0)
     w, b = _rand(96, seed=1), _rand(96, seed=2)
@@ -83,7 +97,7 @@ def test_norm_constant_row_gives_bias(K):
 LINEAR_SHAPES = [(1, 64, 192), (2, 96, 320), (7, 320, 96), (16, 64, 1000), (9, 4104, 200), (12, 1096, 8200), (5, 520, 16400),
                  (17, 96, 50257 // 16), (24, 200, 8200), (21, 1096, 16400), (25, 96, 300), (64, 4096, 528), (65, 256, 257), (130, 96, 300), (300, 1600, 520),
                  (257, 64, 50257 // 8), (520, 72, 33000),
-                 (300, 72, 12288), (300, 1032, 22002)]  # the last four take the 128x128, 256x256, 256x128 and 256x192 tiles
+                 (300, 72, 12288), (300, 1032, 22002), (2048, 64, 6144), (256, 6144, 96)]  # the last four take the 128x128, 256x256, 256x128 and 256x192 tiles
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
