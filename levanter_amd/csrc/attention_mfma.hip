@@ -407,49 +407,96 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   for (int i = 0; i < NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
+  // Every load below is unconditional, from a clamped address, and what it must not deliver is masked out afterwards:
+  // a load under a condition becomes a branch, and at the join the compiler waits for all loads in flight, which
+  // turned the 38 loads of a block into as many round trips to memory, one after the other.
+  // This lane's rows of the token's new value, read once, two to a register.
+  uint32_t nv2[(NDT + 1) / 2];
+#pragma unroll
+  for (int i = 0; i < (NDT + 1) / 2; ++i) nv2[i] = 0u;
+  if (fused) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) nv2[dt / 2] |= (uint32_t)vn[16 * dt + fr] << (16 * (dt & 1));
+  }
+  // Page ids of a block of 64 keys, per lane: one per key tile (u, hh) and one per group of 8 values (u). They are read
+  // one block ahead (behind the block's own loads, into the registers those have just used), so that no key or value
+  // load waits for a table lookup. Positions beyond the token's own are clamped to it (its table entry exists);
+  // vector loads on purpose (the index is made opaque).
+  int kpg[2][2], vpg[2];
+  auto page_ids = [&](int kb) {
+    const int key0 = kb * 64;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        int at = min(key0 + tile_key(u, hh, fr), pos) >> ps_shift;
+        asm volatile("" : "+v"(at));
+        kpg[u][hh] = bt[at];
+      }
+      int at = min(key0 + 32 * u + 8 * g, pos) >> ps_shift;
+      asm volatile("" : "+v"(at));
+      vpg[u] = bt[at];
+    }
+  };
+  page_ids(min(kb_begin, kb_last));
   for (int kb = kb_begin; kb < kb_end; ++kb) {
     const int key0 = kb * 64;
     // key operands: tile (u, hh), row fr is key tile_key(u, hh, fr)
     u32x4 kf[2][2][NKS];
+    uint32_t k_mask[2][2];  // all ones where the key is in the range
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const int kp = key0 + tile_key(u, hh, fr);
-        const bool ok = kp <= pos && kp >= lo;
         const bool is_new = fused && kp == pos;
-        const int page = ok ? bt[kp >> ps_shift] : -1;
-        const bf16_t* base = is_new ? kn : k_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (size_t)(kp & ps_mask) * 8;
+        const int page = kpg[u][hh];
+        k_mask[u][hh] = (kp <= pos && kp >= lo && (page >= 0 || is_new)) ? 0xffffffffu : 0u;
+        const bf16_t* base = is_new ? kn : k_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + (size_t)(kp & ps_mask) * 8;
         const size_t cstride = is_new ? 8 : (size_t)PS * 8;
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
-          const int c = 4 * s + g;
-          kf[u][hh][s] = (page >= 0 && c < NCHUNK) ? *reinterpret_cast<const u32x4*>(base + (size_t)c * cstride) : u32x4{0, 0, 0, 0};
+          const int c = min(4 * s + g, NCHUNK - 1);
+          kf[u][hh][s] = *reinterpret_cast<const u32x4*>(base + (size_t)c * cstride);
         }
       }
     // value operands: tile dt, row fr is head dim 16*dt + fr, k-slots are keys 32u + 8g .. +7
     u32x4 vf[NDT][2];
+    uint32_t v_mask[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int kp = key0 + 32 * u + 8 * g;
-      const bool ok = kp <= pos && kp + 7 >= lo;
-      const int page = ok ? bt[kp >> ps_shift] : -1;
-      const bf16_t* base = v_pages + ((size_t)(page >= 0 ? page : 0) * KVH + kvh) * head_elems + (kp & ps_mask);
-      const int jn = pos - kp;  // slot of the new value among this lane's 8 keys, if 0 <= jn < 8
+      const int page = vpg[u];
+      v_mask[u] = (kp <= pos && kp + 7 >= lo && page >= 0) ? 0xffffffffu : 0u;
+      const bf16_t* base = v_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + (kp & ps_mask);
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) vf[dt][u] = *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS);
+    }
+    page_ids(kb + 1);
+    // what the loads must not deliver: keys outside the range and chunks beyond the head size become zero
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          const uint32_t mk = 4 * s + g < NCHUNK ? k_mask[u][hh] : 0u;
+          kf[u][hh][s] = kf[u][hh][s] & u32x4{mk, mk, mk, mk};
+        }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int jn = pos - (key0 + 32 * u + 8 * g);  // slot of the new value among this lane's 8 keys, if 0 <= jn < 8
       const bool has_new = fused && jn >= 0 && jn < 8;
+      const int w = jn >> 1;
+      // the new value replaces one half of word w: keep-mask and shift of that half
+      const uint32_t keep = (jn & 1) ? 0x0000ffffu : 0xffff0000u;
+      const int shift = (jn & 1) ? 16 : 0;
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
-        u32x4 v = page >= 0 ? *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS) : u32x4{0, 0, 0, 0};
-        if (has_new) {
-          const uint32_t nv = vn[16 * dt + fr];
-          const int w = jn >> 1;
-          const uint32_t old = w == 0 ? v[0] : (w == 1 ? v[1] : (w == 2 ? v[2] : v[3]));
-          const uint32_t neu = (jn & 1) ? ((old & 0x0000ffffu) | (nv << 16)) : ((old & 0xffff0000u) | nv);
-          v[0] = w == 0 ? neu : v[0];
-          v[1] = w == 1 ? neu : v[1];
-          v[2] = w == 2 ? neu : v[2];
-          v[3] = w == 3 ? neu : v[3];
-        }
+        u32x4 v = vf[dt][u] & u32x4{v_mask[u], v_mask[u], v_mask[u], v_mask[u]};
+        const uint32_t nvd = (nv2[dt / 2] >> (16 * (dt & 1))) & 0xffffu;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (has_new && w == e) ? ((v[e] & keep) | (nvd << shift)) : v[e];
         vf[dt][u] = v;
       }
     }
