@@ -97,7 +97,8 @@ __device__ __forceinline__ void tile_epilogue(const f32x16 (&acc)[TI][TJ], float
         }
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = lev_activate_as<ACT>(v[e], act);
+      for (int e = 0; e < 4; ++e)  // the exact GELU of a bfloat16 output takes the short erf
+        v[e] = (ACT == LEV_ACT_GELU_ERF && sizeof(TO) == 2) ? lev_gelu_erf_coarse(v[e]) : lev_activate_as<ACT>(v[e], act);
       if (residual) {
         const float* rrow = residual + (size_t)m * ldr;
         if (whole) {
@@ -270,7 +271,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   }
   if (kt < nk) ktile(kt, 1);
 
-  // Epilogue (the operand buffers are free now), specialised for the two activations that matter so that the
+  // Epilogue (the operand buffers are free now), specialised for no activation and the two GELUs so that the
   // loop over the outputs has no switch inside
   lds_barrier();
   float* Cs = reinterpret_cast<float*>(smem) + wave * 32 * (BN / 2 + 4);
@@ -279,6 +280,8 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
     tile_epilogue<TO, LEV_ACT_NONE, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
   else if (act == LEV_ACT_GELU_TANH)
     tile_epilogue<TO, LEV_ACT_GELU_TANH, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+  else if (act == LEV_ACT_GELU_ERF)
+    tile_epilogue<TO, LEV_ACT_GELU_ERF, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
   else
     tile_epilogue<TO, -1, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
 }
