@@ -2,6 +2,7 @@
 //   y = act(a . w^T + bias) (+ residual),  a [M, K] (row stride lda), w [N, K], y [M, N] bf16 or f32.
 // Three kernels, chosen by M:
 //   tile kernel   (M > 128): a 256x256, 256x192, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
+//                 (K split into ranges, with a second kernel for the sums, where the tiles alone would leave CUs idle)
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
 //   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
 //                 straight into MFMA operand registers, K is split over workgroups and a second kernel
@@ -125,7 +126,7 @@ template <typename TO, int BM, int BN>
 __global__ void __launch_bounds__(256)
 gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                  const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act, int tiles_m, int tiles_n,
-                 int vec_ok) {
+                 int vec_ok, int S, float* __restrict__ partial) {
   constexpr int WM = BM / 2, WN = BN / 2;    // the wave's tile
   constexpr int TI = WM / 32, TJ = WN / 32;  // in 32 x 32 MFMA tiles
   constexpr int CA = BM * (TK / 8) / 256;    // 16-byte chunks of the a tile per thread
@@ -150,11 +151,16 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   for (int i = 0; i < CA; ++i) pa[i] = (uint32_t)((size_t)min(m0 + ((tid + 256 * i) >> 3), M - 1) * lda);
 #pragma unroll
   for (int i = 0; i < CW; ++i) pw[i] = (uint32_t)((size_t)min(n0 + ((tid + 256 * i) >> 3), N - 1) * K);
-  const int ktail = K % TK, nk = (K + TK - 1) / TK;
-  // k offset of tile t (tiles past the end repeat the last one; they are loaded but never used)
+  // The k-tiles in the order they are taken: tile 0 is the partial one (K % 64 != 0) or the first, tile t >= 1 starts at
+  // (t - kshift) * 64. With S > 1 (few output tiles: the K range is split over blockIdx.y) this workgroup takes
+  // tiles t0 .. t1 - 1 and leaves its sums, without epilogue, in partial[blockIdx.y].
+  const int ktail = K % TK, nk_all = (K + TK - 1) / TK;
+  const int per = (nk_all + S - 1) / S;
+  const int t0 = blockIdx.y * per, t1 = min(nk_all, t0 + per);
+  const int nk = t1 - t0;
   const int kshift = ktail ? 1 : 0;
-  auto kpos = [&](int t) {  // for t >= 1; tile 0 starts at K - ktail when there is a partial tile, else at 0
-    return max(min(t, nk - 1) - kshift, 0) * TK;
+  auto kpos = [&](int t) {  // for t >= 1 (tiles past this range repeat its last one; they are loaded but never used)
+    return max(min(t, t1 - 1) - kshift, 0) * TK;
   };
   u32x4 ra[2][CA], rw[2][CW];
   auto gload_one = [&](int set, uint32_t koff, int i) {
@@ -176,8 +182,8 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  {  // prologue: tile 0 (masked in k) to LDS buffer 0, tile 1 into register set 1
-    const int k0 = ktail ? K - ktail : 0;
+  {  // prologue: this range's first tile (masked in k if it is the partial one) to LDS buffer 0, the next into register set 1
+    const int k0 = t0 == 0 ? (ktail ? K - ktail : 0) : kpos(t0);
     const bool ok = k0 + kc < K;
     const uint32_t koff = (uint32_t)min(k0 + kc, K - 8);
 #pragma unroll
@@ -188,7 +194,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
     for (int i = 0; i < CW; ++i) if (!ok) rw[0][i] = u32x4{0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < CA + CW; ++i) lstore_one(0, 0, i);
-    const uint32_t koff1 = (uint32_t)min(kpos(1) + kc, K - 8);
+    const uint32_t koff1 = (uint32_t)min(kpos(t0 + 1) + kc, K - 8);
 #pragma unroll
     for (int i = 0; i < CA + CW; ++i) gload_one(1, koff1, i);
   }
@@ -211,7 +217,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   // most two other instructions so that the matrix pipe never waits for the wave to issue them in a block.
   auto ktile = [&](int kt, int cur) {
     const int buf = kt & 1;
-    const uint32_t koff = (uint32_t)min(kpos(kt + 2) + kc, K - 8);
+    const uint32_t koff = (uint32_t)min(kpos(t0 + kt + 2) + kc, K - 8);
     const bf16_t* Ab = a_rd + buf * BM * LDS_STRIDE;
     const bf16_t* Wb = w_rd + buf * BN * LDS_STRIDE;
     const bf16_t* Abn = a_rd + (buf ^ 1) * BM * LDS_STRIDE;
@@ -276,19 +282,27 @@ gemm_tile_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restric
   lds_barrier();
   float* Cs = reinterpret_cast<float*>(smem) + wave * 32 * (BN / 2 + 4);
   const int mw = m0 + wm * WM, nw = n0 + wn * WN;
-  if (act == LEV_ACT_NONE)
-    tile_epilogue<TO, LEV_ACT_NONE, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+  if (S > 1)  // vec_ok: bit 1 says whether the partial sums can be stored as vectors
+    tile_epilogue<float, LEV_ACT_NONE, TI, TJ>(acc, Cs, lane, mw, nw, nullptr, nullptr, 0, partial + (size_t)blockIdx.y * M * N, N, M, N,
+                                               LEV_ACT_NONE, (vec_ok >> 1) & 1);
+  else if (act == LEV_ACT_NONE)
+    tile_epilogue<TO, LEV_ACT_NONE, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok & 1);
   else if (act == LEV_ACT_GELU_TANH)
-    tile_epilogue<TO, LEV_ACT_GELU_TANH, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+    tile_epilogue<TO, LEV_ACT_GELU_TANH, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok & 1);
   else if (act == LEV_ACT_GELU_ERF)
-    tile_epilogue<TO, LEV_ACT_GELU_ERF, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+    tile_epilogue<TO, LEV_ACT_GELU_ERF, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok & 1);
   else
-    tile_epilogue<TO, -1, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok);
+    tile_epilogue<TO, -1, TI, TJ>(acc, Cs, lane, mw, nw, bias, residual, ldr, out, ldo, M, N, act, vec_ok & 1);
 }
+
+// out = act(sum_s partial[s] + bias) + residual (defined with the stream kernel below)
+template <typename TO>
+static int launch_splitk_reduce(const float* workspace, const float* bias, const float* residual, long ldr, TO* out, long ldo, int M,
+                                int N, int S, int act, hipStream_t stream);
 
 template <typename TO, int BM, int BN>
 static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
-                       long ldo, int M, int N, int K, int act, hipStream_t stream) {
+                       long ldo, float* workspace, int M, int N, int K, int act, int S, hipStream_t stream) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds_ops = (size_t)2 * (BM + BN) * LDS_STRIDE * sizeof(bf16_t);
   const size_t lds_out = (size_t)4 * 32 * (BN / 2 + 4) * sizeof(float);
@@ -299,11 +313,18 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
     if (e != hipSuccess) return lev_fail("linear: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured = true;
   }
+  if (S > 1 && !workspace) return lev_fail("linear: M=%d N=%d K=%d needs a workspace of lev_linear_mfma_workspace bytes", M, N, K);
   // rows of 4 outputs are stored (and bias / residual read) as vectors when everything is aligned for it
-  const int vec_ok = (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) &&
-                     (!bias || ((uintptr_t)bias & 15) == 0);
-  gemm_tile_kernel<TO, BM, BN><<<tiles_m * tiles_n, 256, lds, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act,
-                                                                        tiles_m, tiles_n, vec_ok);
+  const int vec_out = (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) &&
+                      (!bias || ((uintptr_t)bias & 15) == 0);
+  const int vec_partial = (N % 4 == 0) && (((uintptr_t)workspace & 15) == 0);
+  gemm_tile_kernel<TO, BM, BN><<<dim3(tiles_m * tiles_n, S), 256, lds, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act,
+                                                                                   tiles_m, tiles_n, vec_out | (vec_partial << 1), S,
+                                                                                   workspace);
+  if (S > 1) {
+    if (int rc = lev_check_launch("linear_tile")) return rc;
+    return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
+  }
   return 0;
 }
 
@@ -601,6 +622,20 @@ splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict_
   }
 }
 
+template <typename TO>
+static int launch_splitk_reduce(const float* workspace, const float* bias, const float* residual, long ldr, TO* out, long ldo, int M,
+                                int N, int S, int act, hipStream_t stream) {
+  const size_t total = (size_t)M * N;
+  const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (((uintptr_t)workspace & 15) == 0) &&
+                   (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) && (!bias || ((uintptr_t)bias & 15) == 0);
+  if (vec)
+    splitk_reduce_kernel<TO, 1><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo, M, N, S,
+                                                                                          act);
+  else
+    splitk_reduce_kernel<TO, 0><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo, M, N, S, act);
+  return lev_check_launch("linear_reduce");
+}
+
 // Into how many k ranges the stream kernel splits K. Three things are weighed against each other, each relative to
 // the time of streaming the weights once:
 //   balance: the workgroups (column tiles x ranges) go over 256 CUs in rounds, and the last round should be full.
@@ -626,9 +661,50 @@ static int stream_splits(int M, int N, int K) {
   return best;
 }
 
+// Tile shape and number of k ranges for M > 128. Estimated time of each tile shape: rounds of workgroups over the 256
+// CUs times (k-tiles x the shape's time per k-tile + a fixed cost for a tile's first loads and its epilogue). Two
+// 128 x 128 workgroups fit a CU and then share it; up to 256 of them have a CU each. Where the output has so few
+// tiles that most CUs would idle (a few hundred rows times a narrow weight), K is split into ranges, as in the
+// stream kernel: the second kernel then costs its launch and the traffic of the partial sums. The constants are
+// microseconds measured on MI355X.
+struct TilePlan {
+  int shape;   // 0: 256 x 256, 1: 256 x 192, 2: 256 x 128, 3: 128 x 128
+  int splits;  // k ranges (1: none)
+};
+static TilePlan plan_tiles(int M, int N, int K) {
+  static const int bm[4] = {256, 256, 256, 128}, bn[4] = {256, 192, 128, 128};
+  static const double us_per_ktile[4] = {1.72, 1.36, 0.97, 0.6}, fixed[4] = {13.0, 11.0, 9.0, 7.0};
+  const long nk = (K + TK - 1) / TK;
+  TilePlan best = {0, 1};
+  double best_cost = 1e30;
+  for (int i = 0; i < 4; ++i) {
+    const long tiles = (long)((M + bm[i] - 1) / bm[i]) * ((N + bn[i] - 1) / bn[i]);
+    double cost;
+    if (i == 3 && tiles > 256)
+      cost = (double)((tiles + 511) / 512) * (nk * 1.05 + 9.0);
+    else
+      cost = (double)((tiles + 255) / 256) * (nk * us_per_ktile[i] + fixed[i]);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = {i, 1};
+    }
+    for (int s = 2; s <= 16 && tiles * s <= 256 && nk / s >= 4; ++s) {
+      const long per = (nk + s - 1) / s;
+      if (per * (s - 1) >= nk) continue;  // a range would be empty
+      const double reduce = 4.0 + (double)(s + 1) * M * N * 4.0 / 3.0e6;
+      const double c = per * us_per_ktile[i] + fixed[i] + reduce;
+      if (c < best_cost) {
+        best_cost = c;
+        best = {i, s};
+      }
+    }
+  }
+  return best;
+}
+
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
-  if (M <= SKINNY_MAX_M || M > 128) return 0;
-  const int S = stream_splits(M, N, K);
+  if (M <= SKINNY_MAX_M) return 0;
+  const int S = M <= 128 ? stream_splits(M, N, K) : plan_tiles(M, N, K).splits;
   return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
 }
 
@@ -647,18 +723,7 @@ static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float
   else
     gemm_stream_kernel<TO, 8><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
   if (int rc = lev_check_launch("linear_stream")) return rc;
-  if (S > 1) {
-    const size_t total = (size_t)M * N;
-    const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && (((uintptr_t)out & 15) == 0) && (((uintptr_t)workspace & 15) == 0) &&
-                     (!residual || (ldr % 4 == 0 && ((uintptr_t)residual & 15) == 0)) && (!bias || ((uintptr_t)bias & 15) == 0);
-    if (vec)
-      splitk_reduce_kernel<TO, 1><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo,
-                                                                                            M, N, S, act);
-    else
-      splitk_reduce_kernel<TO, 0><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, bias, residual, ldr, out, ldo, M,
-                                                                                        N, S, act);
-    return lev_check_launch("linear_reduce");
-  }
+  if (S > 1) return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
   return 0;
 }
 
@@ -672,28 +737,16 @@ static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const f
   } else {
     if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
       return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
-    // Estimated time of each tile shape: rounds of workgroups over the 256 CUs times (k-tiles x the shape's time per
-    // k-tile + a fixed cost for a tile's first loads and its epilogue). Two 128 x 128 workgroups fit a CU and then
-    // share it; up to 256 of them have a CU each. The constants are microseconds measured on MI355X.
-    const long nk = (K + TK - 1) / TK;
-    auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    auto estimate = [&](int bm, int bn, double us_per_ktile, double fixed) {
-      return (double)((tiles(bm, bn) + 255) / 256) * (nk * us_per_ktile + fixed);
-    };
-    const double e[4] = {estimate(256, 256, 1.72, 13.0), estimate(256, 192, 1.36, 11.0), estimate(256, 128, 0.97, 9.0),
-                         tiles(128, 128) <= 256 ? nk * 0.6 + 7.0 : (double)((tiles(128, 128) + 511) / 512) * (nk * 1.05 + 9.0)};
-    int best = 0;
-    for (int i = 1; i < 4; ++i)
-      if (e[i] < e[best]) best = i;
+    const TilePlan plan = plan_tiles(M, N, K);
     int rc;
-    if (best == 0)
-      rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
-    else if (best == 1)
-      rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
-    else if (best == 2)
-      rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+    if (plan.shape == 0)
+      rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+    else if (plan.shape == 1)
+      rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+    else if (plan.shape == 2)
+      rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
     else
-      rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
+      rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
     if (rc) return rc;
   }
   return lev_check_launch("linear_mfma");
