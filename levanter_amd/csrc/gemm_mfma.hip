@@ -1,7 +1,7 @@
 // bfloat16 matrix products on the matrix cores (MFMA), 32-bit accumulation, fused epilogue:
 //   y = act(a . w^T + bias) (+ residual),  a [M, K] (row stride lda), w [N, K], y [M, N] bf16 or f32.
 // Three kernels, chosen by M:
-//   tile kernel   (M > 128): a 256x256, 256x192, 256x128 or 128x128 tile per workgroup of 4 waves, 32x32x16 MFMA,
+//   tile kernel   (M > 128): a 256x256, 256x192, 256x128, 128x128 or 128x64 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 (K split into ranges, with a second kernel for the sums, where the tiles alone would leave CUs idle)
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
 //   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
@@ -668,19 +668,21 @@ static int stream_splits(int M, int N, int K) {
 // stream kernel: the second kernel then costs its launch and the traffic of the partial sums. The constants are
 // microseconds measured on MI355X.
 struct TilePlan {
-  int shape;   // 0: 256 x 256, 1: 256 x 192, 2: 256 x 128, 3: 128 x 128
+  int shape;   // 0: 256 x 256, 1: 256 x 192, 2: 256 x 128, 3: 128 x 128, 4: 128 x 64
   int splits;  // k ranges (1: none)
 };
 static TilePlan plan_tiles(int M, int N, int K) {
-  static const int bm[4] = {256, 256, 256, 128}, bn[4] = {256, 192, 128, 128};
-  static const double us_per_ktile[4] = {1.72, 1.36, 0.97, 0.6}, fixed[4] = {13.0, 11.0, 9.0, 7.0};
+  static const int bm[5] = {256, 256, 256, 128, 128}, bn[5] = {256, 192, 128, 128, 64};
+  static const double us_per_ktile[5] = {1.72, 1.36, 0.97, 0.6, 0.4}, fixed[5] = {13.0, 11.0, 9.0, 7.0, 6.0};
   const long nk = (K + TK - 1) / TK;
   TilePlan best = {0, 1};
   double best_cost = 1e30;
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 5; ++i) {
     const long tiles = (long)((M + bm[i] - 1) / bm[i]) * ((N + bn[i] - 1) / bn[i]);
     double cost;
-    if (i == 3 && tiles > 256)
+    if (i == 4 && tiles > 256)
+      continue;  // the small tile is for outputs that would leave CUs idle otherwise
+    else if (i == 3 && tiles > 256)
       cost = (double)((tiles + 511) / 512) * (nk * 1.05 + 9.0);
     else
       cost = (double)((tiles + 255) / 256) * (nk * us_per_ktile[i] + fixed[i]);
@@ -745,8 +747,10 @@ static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const f
       rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
     else if (plan.shape == 2)
       rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
-    else
+    else if (plan.shape == 3)
       rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+    else
+      rc = launch_tile<TO, 128, 64>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
     if (rc) return rc;
   }
   return lev_check_launch("linear_mfma");
