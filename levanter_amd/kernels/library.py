@@ -86,6 +86,7 @@ class HipKernels:
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
         self._sample_ws = None
         self._units = {}
+        self._ws, self._ws_outgrown, self._ws_need = {}, [], {}  # GEMM scratch memory per device, see _workspace
         L.lev_attention_prefill_tile_rows.restype = c_int
         self.prefill_tile_rows = int(L.lev_attention_prefill_tile_rows())
 
@@ -159,32 +160,57 @@ class HipKernels:
                                       _DT[out.dtype], _stream()))
 
     # ---- linear ----------------------------------------------------------------------------
+    def _workspace(self, need: int, device) -> torch.Tensor:
+        """Scratch memory for partial sums: one buffer per device that only grows. Kernels on one stream take turns
+        with it. A buffer that is outgrown stays alive, because recorded HIP graphs may point at it; while a graph is
+        being recorded a buffer that is too small is not replaced but a fresh one handed out, which stays with the graph."""
+        ws = self._ws.get(device)
+        if ws is not None and ws.numel() >= need:
+            return ws
+        if torch.cuda.is_current_stream_capturing():
+            return torch.empty(need, dtype=torch.uint8, device=device)
+        if ws is not None:
+            self._ws_outgrown.append(ws)
+        new = torch.empty(max(need, 2 * (ws.numel() if ws is not None else 0)), dtype=torch.uint8, device=device)
+        self._ws[device] = new
+        return new
+
     def linear(self, a, w, bias, out, activation: str = "none", residual=None) -> None:
         """out = act(a @ w.T + bias) (+ residual). a [M, K], w [N, K], out [M, N]; residual float32, may be ``out``."""
-        _dev(a, w, bias, out, residual)
+        # one kernel launch per call: the checks are written to cost little
+        if not (a.is_cuda and w.is_cuda and out.is_cuda and (bias is None or bias.is_cuda) and (residual is None or residual.is_cuda)):
+            raise KernelError("a kernel was given a tensor that is not on the GPU")
         M, K = a.shape
         N = w.shape[0]
-        _req(w.dim() == 2 and w.shape[1] == K and w.is_contiguous(), f"linear: weight must be contiguous [N, {K}]")
-        _req(a.dtype == w.dtype and a.dtype in _DT, "linear: a and w must share a compute dtype")
-        _req(out.shape[0] == M and out.shape[1] == N and out.dtype in _DT, "linear: bad out")
-        _req(a.dtype == torch.bfloat16 or out.dtype == torch.float32, "linear: float32 inputs give float32 outputs")
-        _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()), "linear: bias must be float32 [N]")
+        adt, odt = a.dtype, out.dtype
+        if not (w.dim() == 2 and w.shape[1] == K and w.is_contiguous()):
+            raise KernelError(f"linear: weight must be contiguous [N, {K}]")
+        if not (adt == w.dtype and adt in _DT):
+            raise KernelError("linear: a and w must share a compute dtype")
+        if not (out.shape[0] == M and out.shape[1] == N and odt in _DT):
+            raise KernelError("linear: bad out")
+        if not (adt == torch.bfloat16 or odt == torch.float32):
+            raise KernelError("linear: float32 inputs give float32 outputs")
+        if bias is not None and not (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()):
+            raise KernelError("linear: bias must be float32 [N]")
         lda, ldo = _rows(a, "linear: a"), _rows(out, "linear: out")
         ldr = 0
         if residual is not None:
-            _req(residual.dtype == torch.float32 and residual.shape == out.shape and out.dtype == torch.float32,
-                 "linear: a residual needs a float32 output of its shape")
-            ldr = _rows(residual, "linear: residual")
+            if not (residual.dtype == torch.float32 and residual.shape == out.shape and odt == torch.float32):
+                raise KernelError("linear: a residual needs a float32 output of its shape")
+            ldr = ldo if residual is out else _rows(residual, "linear: residual")
         act = ACTIVATIONS[activation]
-        if a.dtype == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
+        if adt == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
             gemm = self._unit("gemm_mfma")
-            need = gemm.lev_linear_mfma_workspace(M, N, K)  # partial sums of a K range split over workgroups
-            ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need > 0 else None
+            need = self._ws_need.get((M, N, K))
+            if need is None:  # partial sums of a K range split over workgroups
+                need = self._ws_need[(M, N, K)] = gemm.lev_linear_mfma_workspace(M, N, K)
+            ws = self._workspace(need, a.device) if need > 0 else None
             self._check(gemm.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
-                                                 M, N, K, act, _DT[out.dtype], _stream()))
+                                             M, N, K, act, _DT[odt], _stream()))
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
-                                                   M, N, K, act, _DT[a.dtype], _DT[out.dtype], _stream()))
+                                                   M, N, K, act, _DT[adt], _DT[odt], _stream()))
 
     # ---- cache write -----------------------------------------------------------------------
     def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int) -> None:
