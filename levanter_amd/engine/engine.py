@@ -31,8 +31,8 @@ class _Launched:
     """A step that runs on the GPU: its plan, its sampling under way, and whether its sampled tokens can feed the
     next step on the device (every entry one decoded token that wants logits)."""
 
-    def __init__(self, plan, sample, feeds: bool):
-        self.plan, self.sample, self.feeds = plan, sample, feeds
+    def __init__(self, plan, sample):
+        self.plan, self.sample = plan, sample
 
 
 class InferenceEngine:
@@ -112,11 +112,12 @@ class InferenceEngine:
         """Commit one step: plan it and run it (unless it was launched ahead already), sample, append the tokens.
         Returns the sequences that finished in it.
 
-        Decoding is pipelined: while the GPU runs a step of single tokens, the step after it is planned and launched
-        with its token ids taken from the sampler's output on the device, and only then are the first step's tokens
-        read back. The GPU never waits for the host between two decode steps. What cannot be known without the tokens
-        (a stop sequence that ends a request) is settled afterwards: the request's row of the step launched ahead is
-        ignored, and what that row wrote lies in pages that its request no longer owns and nobody reads."""
+        Steps are pipelined: while the GPU runs a step, the step after it is planned from what the host knows
+        (prompt portions, admissions, which requests will decode) and launched with the decoded token ids taken from
+        the sampler's output on the device, and only then are the first step's tokens read back. The GPU does not wait
+        for the host between steps. What cannot be known without the tokens (a stop sequence that ends a request) is
+        settled afterwards: the request's row of the step launched ahead is ignored, and what that row wrote lies in
+        pages that its request no longer owns and nobody reads."""
         pend = self._pending
         self._pending = None
         if pend is None:
@@ -125,10 +126,10 @@ class InferenceEngine:
                 return []
             pend = self._launch(plan, None)
         nxt = None
-        if self.config.decode_lookahead and pend.feeds:
+        if self.config.decode_lookahead:
             ahead = self.scheduler.plan_lookahead(pend.plan)
             if ahead is not None:
-                nxt = self._launch(ahead[0], (pend.sample.tokens, ahead[1]))
+                nxt = self._launch(ahead[0], (pend.sample.tokens, ahead[1]) if ahead[1] else None)
         toks, lps = ([], []) if pend.sample is None else self.sampler.read(pend.sample)
         finished = self.scheduler.commit(pend.plan, toks, lps)
         if nxt is not None:
@@ -159,8 +160,7 @@ class InferenceEngine:
         self.stats["steps"] += 1
         self.stats["tokens_in"] += sum(len(e.tokens) for e in plan)
         self.stats["device_s"] += time.perf_counter() - t0
-        feeds = bool(plan) and all(e.wants_logits and len(e.tokens) == 1 for e in plan)
-        return _Launched(plan, sample, feeds)
+        return _Launched(plan, sample)
 
     def generate(self, requests: Sequence[Request]) -> GenerationResult:
         seqs = self.enqueue_requests(requests)

@@ -21,7 +21,7 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, List, Optional, Sequence, Tuple
+from typing import Dict, Deque, List, Optional, Sequence, Tuple
 
 from levanter_amd.cache import CacheManager, SequenceHandle
 from levanter_amd.config import InferenceEngineConfig
@@ -145,7 +145,8 @@ class Scheduler:
                 continue
             self._preempt(victim)
 
-    def _pick(self) -> Tuple[List[PlannedEntry], bool]:
+    def _taker(self):
+        """take(seq, n): count the pages that n more tokens of seq need against what the pools have left."""
         free = [g.pool.n_free for g in self.cache.groups]
 
         def take(seq: Sequence_, n: int) -> bool:
@@ -156,15 +157,11 @@ class Scheduler:
                 free[i] -= nd
             return True
 
-        entries: List[PlannedEntry] = []
-        starved = False
-        decoding = [s for s in self.running if s.n_cached >= s.prompt_len and s.n_pending == 1]
-        decoding.sort(key=lambda s: s.order)
-        for seq in decoding[: self.cfg.imputed_max_tokens_per_round]:
-            if take(seq, 1):
-                entries.append(PlannedEntry(seq, [seq.tokens[-1]], True))
-            else:
-                starved = True
+        return take, free
+
+    def _pick_portions(self, entries: List[PlannedEntry], take, free) -> bool:
+        """Prompt portions under the token budget, oldest request first, behind the entries already picked.
+        Returns whether the step is starved (nothing picked at all because the pages ran out)."""
         budget = self.cfg.imputed_max_prefill_size
         n_prefill = 0
         for seq in sorted((s for s in self.running if s.n_cached < s.prompt_len), key=lambda s: s.order):
@@ -177,40 +174,61 @@ class Scheduler:
                 room = min(free) * ps + (-seq.handle.length) % ps
                 n = min(n - 1, room)
             if n <= 0:
-                if not entries:
-                    starved = True
-                break
+                return not entries
             start = seq.n_cached
             entries.append(PlannedEntry(seq, seq.tokens[start:start + n], start + n == len(seq.tokens)))
             budget -= n
             n_prefill += 1
+        return False
+
+    def _pick(self) -> Tuple[List[PlannedEntry], bool]:
+        take, free = self._taker()
+        entries: List[PlannedEntry] = []
+        starved = False
+        decoding = [s for s in self.running if s.n_cached >= s.prompt_len and s.n_pending == 1]
+        decoding.sort(key=lambda s: s.order)
+        for seq in decoding[: self.cfg.imputed_max_tokens_per_round]:
+            if take(seq, 1):
+                entries.append(PlannedEntry(seq, [seq.tokens[-1]], True))
+            else:
+                starved = True
+        starved = self._pick_portions(entries, take, free) or starved
         return entries, starved
 
     def plan_lookahead(self, pending: List[PlannedEntry]) -> Optional[Tuple[List[PlannedEntry], List[int]]]:
         """The step after ``pending`` (a launched step whose sampled tokens are not on the host yet), if it can be
-        decided without them: ``pending`` is every running request decoding one token, nobody waits for admission,
-        and the pools hold the pages. Requests that end by length with ``pending``'s token are left out; one that
-        ends by a stop sequence cannot be foreseen and is skipped when this step is committed. Returns the entries
-        (their token lists hold a placeholder) and, for each, its row among ``pending``'s entries; None: plan as usual."""
-        if self.waiting or not pending or len(pending) != len(self.running) or len(pending) > self.cfg.imputed_max_tokens_per_round:
+        decided without them. Every request that ``pending`` samples a token for decodes that token next: its entry
+        holds a placeholder, and its row among ``pending``'s sampled tokens is returned beside the entries (these
+        entries come first). Prompt portions and admissions follow as in ``plan``, from what the host knows. Requests
+        that end by length with ``pending``'s token are left out; one that ends by a stop sequence cannot be foreseen
+        and is skipped when this step is committed (so are the pages and the slot it would have given back: the plan is
+        made as if nobody ended). Nothing is preempted here. None: wait for the tokens and plan as usual."""
+        if not pending or any(e.seq.done for e in pending):
             return None
-        if any(not e.wants_logits or len(e.tokens) != 1 or e.seq.done for e in pending):
+        row_of: Dict[int, int] = {}
+        for e in pending:
+            if e.wants_logits:
+                row_of[id(e.seq)] = len(row_of)
+        # a request that decodes a token the host knows would have to stand among the fed ones
+        if any(s.n_cached >= s.prompt_len and s.n_pending == 1 for s in self.running):
             return None
-        free = [g.pool.n_free for g in self.cache.groups]
+        decoders = sorted((s for s in self.running if id(s) in row_of), key=lambda s: s.order)
+        if len(decoders) > self.cfg.imputed_max_tokens_per_round:
+            return None
+        if self._steps_since_admission >= self.cfg.max_rounds or any(s.n_cached < s.prompt_len for s in self.running):
+            self._admit()
+            self._steps_since_admission = 0
+        take, free = self._taker()
         entries: List[PlannedEntry] = []
         rows: List[int] = []
-        for i, e in enumerate(pending):
-            seq = e.seq
+        for seq in decoders:
             if len(seq.tokens) + 1 >= min(seq.request.decode_params.max_num_tokens, self.max_len):
                 continue  # pending's token is its last
-            need = [g.blocks_needed(seq.handle.slot, seq.handle.length, seq.handle.length + 1) for g in self.cache.groups]
-            if any(nd > fr for nd, fr in zip(need, free)):
+            if not take(seq, 1):
                 return None  # pages run out: the ordinary plan decides whom to preempt
-            for k, nd in enumerate(need):
-                free[k] -= nd
             entries.append(PlannedEntry(seq, [0], True))
-            rows.append(i)
-        if not entries:
+            rows.append(row_of[id(seq)])
+        if self._pick_portions(entries, take, free) or not entries:
             return None
         self._steps_since_admission += 1
         return entries, rows

@@ -92,8 +92,8 @@ class ModelRunner:
         """Run the entries as one batch. Returns float32 logits [wanted, vocab] in the order of the
         entries and of their ``want``. Raises ``OutOfPages`` (nothing changed) if a pool is too small.
         ``copy_out=False`` may return a buffer that the next step overwrites (the sampler reads it at once).
-        ``token_feed = (device_tokens int32 [R], rows, n)``: the n entries are single tokens that are not known on the
-        host yet; entry i's token is ``device_tokens[rows[i]]`` (``rows`` None: ``device_tokens[i]``), the sampler's
+        ``token_feed = (device_tokens int32 [R], rows, n)``: the first n entries are single tokens that are not known on
+        the host yet; entry i's token is ``device_tokens[rows[i]]`` (``rows`` None: ``device_tokens[i]``), the sampler's
         output of the step before, put in place on the device after the step's tables have been uploaded."""
         entries = list(entries)
         self._validate(entries)
@@ -107,8 +107,8 @@ class ModelRunner:
             self.cache.extend(e.handle, len(e.tokens))
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
         batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
-        if token_feed is not None and any(len(e.tokens) != 1 for e in entries):
-            raise StepError("tokens can be fed from the device to entries of a single token only")
+        if token_feed is not None and (token_feed[2] > len(entries) or any(len(e.tokens) != 1 for e in entries[:token_feed[2]])):
+            raise StepError("tokens can be fed from the device to the step's first entries only, each of a single token")
         if graphable:
             logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
             if copy_out:
@@ -231,7 +231,7 @@ class ModelRunner:
     # ---- decode steps as HIP graphs --------------------------------------------------------
     @staticmethod
     def _feed_tokens(dev: torch.Tensor, b: "HostBatch", token_feed) -> None:
-        """Entry i's token id comes from ``device_tokens[rows[i]]`` (the entries are the first tokens of the step)."""
+        """Entry i's token id (i < n) comes from ``device_tokens[rows[i]]``: these entries are the step's first tokens."""
         if token_feed is None:
             return
         device_tokens, rows, n = token_feed

@@ -223,3 +223,43 @@ def test_steps_launched_ahead_change_nothing():
     assert with_la[0][0][-2:] == [9, 10] and with_la[0][1] == "stop" and with_la[1][1] == "length"
     # a step launched ahead carried one row too many whenever a stop sequence ended a request: more rows in all, never fewer steps
     assert sum(map(sum, batches_la)) > sum(map(sum, batches)) and len(batches_la) >= len(batches)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_with_prompt_portions_and_admissions_are_launched_ahead_too(seed):
+    """Random requests arriving over time, prompts cut into small portions, few slots and pages: with steps launched
+    ahead (prompt portions and admissions included) every request generates what it generates without, nothing is
+    lost from the pools, and steps really were launched before their predecessor's tokens were read."""
+    import random
+
+    rng = random.Random(seed)
+    n = 14
+    reqs = []
+    for i in range(n):
+        new = rng.choice([1, 2, 6, 15])
+        plen = rng.choice([1, 2, 5, 17, 33, 40])
+        stop = [[rng.randrange(40)], [rng.randrange(40), rng.randrange(40)]] if rng.random() < 0.5 else None
+        reqs.append(dict(prompt_tokens=[rng.randrange(40) for _ in range(plen)], request_id=i, enable_logprobs=True,
+                         decode_params=SeqDecodingParams(max_num_tokens=plen + new, stop_tokens=stop, temperature=rng.choice([0.0, 0.8]))))
+    arrivals = sorted(rng.randrange(0, 30) for _ in range(n)) + [10 ** 9]
+    kw = dict(max_pages=rng.choice([12, 20, 64]), max_seqs=rng.choice([3, 5, 8]), max_prefill_size=rng.choice([5, 16, 64]),
+              max_seqs_in_prefill=rng.choice([1, 4]), enable_logprobs=True)
+
+    def run(lookahead):
+        engine, model = make_engine(DummyModel(vocab_size=40, count=True), decode_lookahead=lookahead, **kw)
+        seqs, pending, step, ahead = [], [Request(**r) for r in reqs], 0, 0
+        while pending or not all(s.done for s in seqs):
+            while pending and arrivals[len(seqs)] <= step:
+                seqs += engine.enqueue_requests([pending.pop(0)])
+            engine.step()
+            ahead += engine._pending is not None
+            step += 1
+            assert step < 5000
+        assert engine._pending is None and all_released(engine)
+        return [(list(s.generated), s.finish_reason, [round(x, 5) for x in s.logprobs]) for s in seqs], ahead, model.batches
+
+    with_la, ahead, batches_la = run(True)
+    without, none_ahead, _ = run(False)
+    assert with_la == without
+    assert none_ahead == 0 and ahead > 0
+    assert any(max(b) > 1 and len(b) > 1 for b in batches_la)  # portions of prompts beside decoded tokens in one step
