@@ -636,23 +636,27 @@ static int launch_splitk_reduce(const float* workspace, const float* bias, const
   return lev_check_launch("linear_reduce");
 }
 
-// Into how many k ranges the stream kernel splits K. Three things are weighed against each other, each relative to
-// the time of streaming the weights once:
-//   balance: the workgroups (column tiles x ranges) go over 256 CUs in rounds, and the last round should be full.
-//     With 192 column tiles 3 ranges give 576 workgroups: a quarter of the CUs takes three, the rest two, and the
-//     kernel lasts as long as with 2 ranges; 4 ranges give three to every CU;
-//   latency: with fewer than two workgroups per CU the loads in flight do not cover the memory latency;
-//   the partial sums: every range writes M x N floats that the second kernel reads again (4 S M / K of the weights'
-//     bytes, but mostly out of the caches: weighted half), and the second launch itself.
+// Into how many k ranges the stream kernel splits K: an estimate in microseconds, fitted to measurements on MI355X
+// of weights from 5 MB to 130 MB at 32 and 64 rows.
+//   The workgroups (column tiles x ranges) go over the 256 CUs in rounds; a round costs about 2 us of its own plus
+//     its share of the time to stream the weights at 4.5 TB/s. With 192 column tiles 3 ranges give 576 workgroups:
+//     a quarter of the CUs takes three, the rest two, and the kernel lasts as long as with 2 ranges; 4 ranges give
+//     three to every CU.
+//   Weights of more than 6 us with fewer than two workgroups per CU: the loads in flight do not cover the memory
+//     latency (x 1.5).
+//   More than one range: the second kernel's launch (3 us) and the partial sums, M x N floats per range that are
+//     written and read again (4 S M / K of the weights' bytes, mostly out of the caches: weighted half).
 static int stream_splits(int M, int N, int K) {
   const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
   const int s_max = chunks / 2 < 16 ? (chunks / 2 < 1 ? 1 : chunks / 2) : 16;  // at least two chunks each
+  const double t_stream = (double)N * K * 2.0 / 4.5e6;
   int best = 1;
   double best_cost = 1e30;
   for (int s = 1; s <= s_max; ++s) {
     const long wgs = (long)tiles * s;
-    const double imbalance = ((double)((wgs + 255) / 256) / s) / (tiles / 256.0);
-    const double cost = imbalance * (wgs < 512 ? 1.5 : 1.0) + (s > 1 ? 0.1 + 2.0 * s * M / K : 0.0);
+    double cost = (double)((wgs + 255) / 256) * (2.0 + t_stream * 256.0 / wgs);
+    if (wgs < 512 && t_stream > 6.0) cost *= 1.5;
+    if (s > 1) cost += 3.0 + 2.0 * s * M / K * t_stream;
     if (cost < best_cost - 1e-9) {
       best_cost = cost;
       best = s;
