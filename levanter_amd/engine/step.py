@@ -97,6 +97,8 @@ class ModelRunner:
         output of the step before, put in place on the device after the step's tables have been uploaded."""
         entries = list(entries)
         self._validate(entries)
+        if token_feed is not None and (token_feed[2] > len(entries) or any(len(e.tokens) != 1 for e in entries[:token_feed[2]])):
+            raise StepError("tokens can be fed from the device to the step's first entries only, each of a single token")
         if not entries:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.env.device)
         if not self.fits(entries):
@@ -107,8 +109,6 @@ class ModelRunner:
             self.cache.extend(e.handle, len(e.tokens))
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
         batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
-        if token_feed is not None and (token_feed[2] > len(entries) or any(len(e.tokens) != 1 for e in entries[:token_feed[2]])):
-            raise StepError("tokens can be fed from the device to the step's first entries only, each of a single token")
         if graphable:
             logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
             if copy_out:

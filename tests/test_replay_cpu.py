@@ -100,3 +100,32 @@ def test_step_refuses_bad_input(setup):
     assert h2.length == 0
     cache.check_invariants()
     assert runner.step([]).shape == (0, raw["vocab_size"])
+
+
+def test_token_ids_from_the_device_for_the_first_entries_of_a_mixed_step(setup):
+    """A step may take the token ids of its first entries (single tokens) from a tensor on the device, in any order
+    of its rows, beside a prompt portion given on the host: the logits equal those of the same step with all ids
+    given; fed ids for an entry of several tokens, or for more entries than the step has, are refused."""
+    raw, model, env, reqs, plain = setup
+    cfg = InferenceEngineConfig(max_pages=32, max_seqs=4, page_size=16, max_pages_per_seq=16, compute_dtype="float32")
+    toks = list(reqs.values())
+
+    def run(feed):
+        cache = make_cache(model, cfg)
+        runner = ModelRunner(model, cache, env)
+        a, b, c = cache.open("a"), cache.open("b"), cache.open("c")
+        runner.step([StepEntry(a, toks[0][:20], []), StepEntry(b, toks[1][:7], [])])
+        ids = [toks[0][20], toks[1][7]]
+        entries = [StepEntry(a, [0] if feed else [ids[0]], [0]), StepEntry(b, [0] if feed else [ids[1]], [0]),
+                   StepEntry(c, toks[2][:9], [8])]
+        if not feed:
+            return runner.step(entries)
+        sampled = torch.tensor([5, ids[1], 7, ids[0]], dtype=torch.int32)  # rows of another step's sampler output
+        with pytest.raises(StepError, match="first entries"):
+            runner.step(entries, token_feed=(sampled, torch.tensor([3, 1, 0]), 3))
+        with pytest.raises(StepError, match="first entries"):
+            runner.step(entries, token_feed=(sampled, torch.tensor([3, 1, 0, 2]), 4))
+        assert a.length == 20 and c.length == 0  # a refused step changes nothing
+        return runner.step(entries, token_feed=(sampled, torch.tensor([3, 1]), 2))
+
+    torch.testing.assert_close(run(True), run(False), rtol=0, atol=0)
