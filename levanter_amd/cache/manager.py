@@ -229,6 +229,18 @@ class CacheManager:
                     g.pool.free(page)
             raise
 
+    def retract(self, h: SequenceHandle, n_new: int) -> None:
+        """Undo an ``extend`` whose tokens were never written (the step failed before it ran): the pages of blocks
+        beyond the request's length go back to their pools."""
+        have = (h.length + self.page_size - 1) // self.page_size
+        want = (h.length + n_new + self.page_size - 1) // self.page_size
+        for g in self.groups:
+            for b in range(have, min(want, g.block_tables.shape[1])):
+                page = int(g.block_tables[h.slot, b])
+                if page != NO_PAGE:
+                    g.block_tables[h.slot, b] = NO_PAGE
+                    g.pool.free(page)
+
     def advance(self, h: SequenceHandle, n_new: int) -> None:
         """The step has written ``n_new`` tokens: count them, give back what windows have passed."""
         h.length += n_new

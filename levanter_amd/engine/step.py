@@ -105,18 +105,25 @@ class ModelRunner:
             need = self.pages_needed(entries)
             raise OutOfPages("out of free pages: the step needs " + ", ".join(
                 f"{n} of group {g.index}'s {g.pool.n_free} free" for n, g in zip(need, self.cache.groups)))
-        for e in entries:
-            self.cache.extend(e.handle, len(e.tokens))
-        graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
-        batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
-        if graphable:
-            logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
-            if copy_out:
-                logits = logits.clone()
-        else:
-            dev = self._upload(batch.host)
-            self._feed_tokens(dev, batch, token_feed)
-            logits = self.model.forward(self._make_ctx(dev, batch, self._workspaces), batch.rows_view)
+        extended: List[StepEntry] = []
+        try:
+            for e in entries:
+                self.cache.extend(e.handle, len(e.tokens))
+                extended.append(e)
+            graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+            batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
+            if graphable:
+                logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
+                if copy_out:
+                    logits = logits.clone()
+            else:
+                dev = self._upload(batch.host)
+                self._feed_tokens(dev, batch, token_feed)
+                logits = self.model.forward(self._make_ctx(dev, batch, self._workspaces), batch.rows_view)
+        except BaseException:  # the step did not happen: its pages go back
+            for e in extended:
+                self.cache.retract(e.handle, len(e.tokens))
+            raise
         for e in entries:
             self.cache.advance(e.handle, len(e.tokens))
         return logits

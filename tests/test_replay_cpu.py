@@ -129,3 +129,30 @@ def test_token_ids_from_the_device_for_the_first_entries_of_a_mixed_step(setup):
         return runner.step(entries, token_feed=(sampled, torch.tensor([3, 1]), 2))
 
     torch.testing.assert_close(run(True), run(False), rtol=0, atol=0)
+
+
+def test_a_step_that_fails_in_the_model_gives_its_pages_back(setup, monkeypatch):
+    raw, model, env, reqs, plain = setup
+    cfg = InferenceEngineConfig(max_pages=16, max_seqs=2, page_size=16, max_pages_per_seq=16, compute_dtype="float32")
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    toks = list(reqs.values())[0]
+    a, b = cache.open("a"), cache.open("b")
+    runner.step([StepEntry(a, toks[:20], [])])
+    free = [g.pool.n_free for g in cache.groups]
+    real_forward = model.forward
+
+    def broken(ctx, rows):
+        raise RuntimeError("a part failed")
+
+    monkeypatch.setattr(model, "forward", broken)
+    with pytest.raises(RuntimeError, match="a part failed"):
+        runner.step([StepEntry(a, toks[20:45], [24]), StepEntry(b, toks[:33], [])])
+    assert a.length == 20 and b.length == 0 and [g.pool.n_free for g in cache.groups] == free
+    cache.check_invariants()
+    monkeypatch.setattr(model, "forward", real_forward)
+    got = runner.step([StepEntry(a, toks[20:45], [24]), StepEntry(b, toks[:33], [])])
+    torch.testing.assert_close(got[0].double(), plain[list(reqs)[0]][44], rtol=1e-4, atol=1e-5)
+    cache.close(a)
+    cache.close(b)
+    assert all(g.pool.n_free == g.pool.n_pages for g in cache.groups)
