@@ -351,8 +351,8 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
 //     the device-scope fences it needs cost several times the second launch.)
 //
 // k_new != null: the step's new key and value of each token are not in the cache yet. The wave whose key
-// range holds the token's own position takes them from k_new / v_new (rows of the projection's output),
-// uses them in place of what the cache holds there, and writes them to dest[t] = page * PS + offset.
+// range holds the token's own position takes them from k_new / v_new (rows of the projection's output) and
+// uses them in place of what the cache holds there; one wave copies them to dest[t] = page * PS + offset.
 #define DECODE_WG_WAVES 8
 __global__ void __launch_bounds__(64 * DECODE_WG_WAVES)
 LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
@@ -379,11 +379,15 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   const int q_pos = fr < G ? pos : -1;
   const size_t head_elems = (size_t)HD << ps_shift;
   const bool fused = k_new != nullptr;
-  const bool owner = fused && kb_begin <= kb_last && kb_last < kb_end;  // this wave's range holds the token's position
+  // The new key and value are copied to their page by one wave of the (token, kv head): the last one if it has no keys
+  // of its own (the ranges are rounded up, so with few blocks the last waves are idle), else the wave whose range
+  // holds the token's position, which then has the copy ahead of its two or more blocks.
+  const bool idle_last = splits > 1 && kb_first + (splits - 1) * per > kb_last;
+  const bool owner = fused && (idle_last ? z == splits - 1 : (kb_begin <= kb_last && kb_last < kb_end));
   const bf16_t* kn = fused ? k_new + (size_t)t * kv_stride + (size_t)kvh * HD : nullptr;
   const bf16_t* vn = fused ? v_new + (size_t)t * kv_stride + (size_t)kvh * HD : nullptr;
 
-  if (owner) {  // the new key and value go to their page (read by later steps only)
+  if (owner) {  // read by later steps only: this step takes them from k_new / v_new
     const int dst = dest[t];
     if (dst >= 0) {
       bf16_t* kb_ = k_pages + ((size_t)(dst >> ps_shift) * KVH + kvh) * head_elems;
