@@ -132,6 +132,44 @@ def test_linear_plain_and_epilogues(K, dtype, M, K_, N):
     torch.testing.assert_close(x.cpu(), want, rtol=2e-5 if dtype == torch.float32 else 1e-3, atol=2e-5 if dtype == torch.float32 else 1e-3)
 
 
+def test_linear_bf16_random_shapes_strides_and_epilogues(K):
+    """Sixty random shapes through the bfloat16 kernels (skinny, stream, tiles of every shape, K split into ranges),
+    with row strides above K, every epilogue and both output types, against the float64 statement."""
+    import random
+
+    rng = random.Random(7)
+    acts = {"none": lambda x: x, "relu": torch.relu, "gelu_new": lambda x: torch.nn.functional.gelu(x, approximate="tanh"),
+            "gelu": torch.nn.functional.gelu, "silu": torch.nn.functional.silu}
+    done = 0
+    while done < 60:
+        M = rng.choice([1, 3, 8, 16, 17, 24, 25, 31, 64, 100, 128, 129, 190, 256, 300, 511, 777, 1024])
+        K_ = 8 * rng.choice([1, 2, 8, 9, 25, 64, 100, 129, 200, 513, 800])
+        N = rng.choice([1, 5, 16, 63, 64, 100, 192, 200, 257, 520, 1000, 1600, 3333, 4800])
+        if M * N > 2_000_000 or N * K_ > 8_000_000:
+            continue
+        done += 1
+        with_res, with_bias = rng.random() < 0.4, rng.random() < 0.7
+        act = "none" if with_res else rng.choice(list(acts))
+        lda = K_ + 8 * rng.choice([0, 0, 1, 3])
+        a = _rand(M, lda, dtype=torch.bfloat16, seed=done).to(DEV)[:, :K_]
+        w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=100 + done).to(DEV)
+        bias = _rand(N, seed=200 + done).to(DEV) if with_bias else None
+        want = a.double() @ w.double().t()
+        if with_bias:
+            want = want + bias.double()
+        want = acts[act](want)
+        if with_res:
+            out = _rand(M, N, seed=300 + done).to(DEV)
+            want = want + out.double()
+            K.linear(a, w, bias, out, residual=out)
+        else:
+            out = torch.full((M, N), float("nan"), device=DEV, dtype=rng.choice([torch.bfloat16, torch.float32]))
+            K.linear(a, w, bias, out, activation=act)
+        tol = 2e-2 if out.dtype == torch.bfloat16 else 2e-3  # of the largest output: bfloat16 operands, float32 sums
+        err = float((out.double() - want).abs().max() / (want.abs().max() + 1e-6))
+        assert err < tol, (M, K_, N, lda, act, with_res, with_bias, out.dtype, err)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_strided_input_and_all_activations(K, dtype):
     M, K_, N = 9, 96, 40
