@@ -268,6 +268,60 @@ def test_paged_attention(K, dtype, H, KVH, HD, PS, runs, window):
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
 
 
+def test_paged_attention_random_cases(K):
+    """Forty random cases in bfloat16: head sizes 16 .. 128, groups of query heads, page sizes, windows, prompt portions
+    beside single tokens. Steps of single tokens also go through the kernel that takes the new key and value from
+    the projection's output: same output and same pages, bit for bit, as writing them first."""
+    import random
+
+    rng = random.Random(11)
+    dtype = torch.bfloat16
+    for trial in range(40):
+        HD = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+        KVH, G = rng.choice([1, 2, 3, 5]), rng.choice([1, 1, 2, 4])
+        H, PS = KVH * G, rng.choice([16, 16, 32, 64])
+        decode_only = rng.random() < 0.4
+        runs = []
+        for _ in range(rng.choice([1, 2, 3, 5])):
+            kv = rng.choice([1, 2, 15, 16, 17, 33, 64, 65, 100, 129, 200, 333, 640])
+            qn = 1 if decode_only or rng.random() < 0.4 else rng.choice([2, 3, 16, 17, 64, 130])
+            runs.append((min(qn, kv), kv))
+        window = rng.choice([None, None, 5, 16, 40, 100])
+        kv_lens = [k for _, k in runs]
+        n_pages = sum((k + PS - 1) // PS for k in kv_lens) + 3
+        case = f"trial {trial}: H={H} KVH={KVH} HD={HD} PS={PS} runs={runs} window={window}"
+        T = sum(q for q, _ in runs)
+        scale = 1 / math.sqrt(HD) / 2
+        args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=scale, window=window)
+        if decode_only and rng.random() < 0.6:
+            bt = random_block_tables(kv_lens, PS, n_pages, 3, "cpu")
+            kd = torch.zeros(n_pages, KVH * HD * PS, dtype=dtype, device=DEV)
+            vd = torch.zeros_like(kd)
+            for s_, n in enumerate(kv_lens):
+                if n > 1:
+                    kk, vv = _rand(n - 1, KVH * HD, dtype=dtype, seed=50 + s_), _rand(n - 1, KVH * HD, dtype=dtype, seed=90 + s_)
+                    K.kv_write(kk.to(DEV), vv.to(DEV), kd, vd, torch.tensor(dest_for(bt, s_, range(n - 1), PS), dtype=torch.int32, device=DEV), KVH, HD, PS)
+            q = _rand(T, H * HD, dtype=dtype, seed=5).to(DEV)
+            k_new, v_new = _rand(T, KVH * HD, dtype=dtype, seed=6).to(DEV), _rand(T, KVH * HD, dtype=dtype, seed=7).to(DEV)
+            dest = torch.tensor([dest_for(bt, s_, [n - 1], PS)[0] for s_, n in enumerate(kv_lens)], dtype=torch.int32, device=DEV)
+            k2, v2 = kd.clone(), vd.clone()
+            K.kv_write(k_new, v_new, k2, v2, dest, KVH, HD, PS)
+            two = torch.empty(T, H * HD, dtype=dtype, device=DEV)
+            K.paged_attention(q, two, k2, v2, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+            got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+            assert K.paged_attention(q, got, kd, vd, make_meta(runs, DEV), k_new=k_new, v_new=v_new, dest=dest, block_tables=bt.to(DEV), **args), case
+            assert torch.equal(got, two) and torch.equal(kd, k2) and torch.equal(vd, v2), case
+            q, kp, vp = q.cpu(), k2.cpu(), v2.cpu()
+        else:
+            bt, kp, vp, kd, vd, _, _ = _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed=7)
+            q = _rand(T, H * HD, dtype=dtype, seed=11)
+            got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+            K.paged_attention(q.to(DEV), got, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+        want = torch.empty(T, H * HD, dtype=dtype)
+        EMU.paged_attention(q, want, kp, vp, make_meta(runs, "cpu"), block_tables=bt, **args)
+        torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2, msg=lambda m: case + "\n" + m)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_one_far_key(K, dtype):
     # among 700 keys one (far back, in the middle of a page) matches the query strongly: the output is its value
