@@ -281,8 +281,12 @@ class HipKernels:
         want = max(1, 2048 // max(1, meta.n_decode * n_kv_heads))
         most = max(1, (meta.max_kv_len + 63) // 64)  # at least 64 keys per split
         splits = int(min(want, most, 64))
-        if splits > 8 and most <= 32:
-            splits = 8  # up to 8 splits are merged inside one workgroup (no second kernel); worth 4 blocks of keys per wave
+        if splits > 8 and most <= 16 and meta.n_decode * n_kv_heads >= 128:
+            # Up to 8 splits are merged inside one workgroup (no second kernel). That is worth two blocks of keys per
+            # wave where the workgroups alone give the chip a few hundred waves; with fewer (one or two requests) a
+            # wave per block and the combine kernel are faster at every context length (measured at 32 heads of 128:
+            # batch 1, 1,850 keys: 3.73 -> 3.26 ms a step; batch 4, 580 keys: 3.39 ms with the clamp, 3.43 without).
+            splits = 8
         return splits
 
     @staticmethod
