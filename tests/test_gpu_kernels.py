@@ -244,6 +244,8 @@ ATTN_CASES = [
     (4, 1, 128, 16, [(1, 300), (130, 260)], 50),
     (3, 3, 32, 16, [(1, 100), (20, 90), (1, 7)], 16),
     (2, 2, 256, 16, [(1, 40), (9, 33)], None),
+    (32, 32, 128, 16, [(1, 1850)], None),  # a lone long request: many key ranges, merged by the combine kernel
+    (6, 2, 64, 16, [(1, 1200), (1, 520)], 600),
 ]
 
 
@@ -391,6 +393,9 @@ def test_sample_ties_and_frequencies(K):
     (4, 4, 64, 16, [1, 17, 64, 65, 300], None),
     (8, 2, 128, 16, [16, 33, 640], None),
     (3, 3, 32, 32, [5, 100, 31, 32, 33], 40),
+    (32, 32, 128, 16, [1850, 40, 7], None),  # few requests, long context: a wave per block of keys, merged by the combine kernel
+    (8, 8, 64, 16, [1000, 2047, 9], None),
+    (4, 2, 96, 16, [1500, 3, 100], 700),
 ])
 def test_decode_attention_that_writes_its_own_keys_and_values(K, H, KVH, HD, PS, kv_lens, window):
     """A step of single tokens may hand the new keys and values to the attention kernel instead of writing
@@ -429,7 +434,10 @@ def test_decode_attention_that_writes_its_own_keys_and_values(K, H, KVH, HD, PS,
     meta2._workspaces = meta._workspaces
     got2 = torch.empty(2, H * HD, dtype=dtype, device=DEV)
     K.paged_attention(q[:2], got2, k2, v2, meta2, **{**args, "block_tables": bt[:2].contiguous().to(DEV)})
-    torch.testing.assert_close(got2.float().cpu(), want[:2].float().cpu(), rtol=0, atol=0)
+    # the same bits where both launches cut the keys into the same ranges; else the sums differ in their rounding
+    same_cut = K.decode_splits(meta2, H, KVH) == K.decode_splits(meta, H, KVH)
+    tol = 0 if same_cut else 1e-2
+    torch.testing.assert_close(got2.float().cpu(), want[:2].float().cpu(), rtol=tol, atol=tol)
     # with prompt portions in the step the kernel declines and the caller writes first
     mixed = make_meta([(2, 10), (1, 5)], DEV)
     assert K.paged_attention(q[:3], got[:3], k2, v2, mixed, k_new=k_new[:3], v_new=v_new[:3], dest=dest[:3], **args) is False
