@@ -507,22 +507,25 @@ gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
     xoff[i] = (uint32_t)((size_t)min(row, M - 1) * lda);
     xlds[i] = row * SK_LDS_STRIDE + xk[i];
   }
-  u32x4 xr[XCH];
+  // two register sets for the a tile as for the weights: a chunk's loads are issued two iterations before it is
+  // stored to LDS. With one set an iteration could not be shorter than the L2 latency of the a loads of the
+  // iteration before (about a microsecond, where its own work is a few hundred cycles).
+  u32x4 xr[2][XCH];
   constexpr int KS = SK_CHUNK / 32;  // k-steps per chunk
   u32x4 wr[2][KS];
-  auto load_x = [&](int c) {
+  auto load_x = [&](int set, int c) {
     const int k0 = min(c, n_chunks - 1) * SK_CHUNK;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       const int k = k0 + xk[i];
-      xr[i] = load16(a + xoff[i] + (k < K ? k : K - 8));
+      xr[set][i] = load16(a + xoff[i] + (k < K ? k : K - 8));
     }
   };
-  auto store_x = [&](int buf, int c) {
+  auto store_x = [&](int buf, int set, int c) {
     const int k0 = c * SK_CHUNK;
 #pragma unroll
     for (int i = 0; i < XCH; ++i)
-      *reinterpret_cast<u32x4*>(&Xs[buf][xlds[i]]) = (k0 + xk[i] < K) ? xr[i] : u32x4{0, 0, 0, 0};
+      *reinterpret_cast<u32x4*>(&Xs[buf][xlds[i]]) = (k0 + xk[i] < K) ? xr[set][i] : u32x4{0, 0, 0, 0};
   };
   auto load_w = [&](int set, int c) {
     const int k0 = min(c, n_chunks - 1) * SK_CHUNK;
@@ -537,19 +540,20 @@ gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   if (c_begin < c_end) {
-    load_x(c_begin);
+    load_x(0, c_begin);
     load_w(0, c_begin);
-    store_x(0, c_begin);
-    load_x(c_begin + 1);
+    load_x(1, c_begin + 1);
     load_w(1, c_begin + 1);
+    store_x(0, 0, c_begin);
+    load_x(0, c_begin + 2);
     lds_barrier();
+    // chunk c (weights in set `set`, a tile in LDS buffer `set`): the a tile of chunk c + 1, in registers since the
+    // iteration before last, goes to the other buffer; its registers are refilled three chunks ahead, this chunk's
+    // weight registers two chunks ahead
     auto chunk = [&](int c, int set) {
-      // the a tile of chunk c + 1 (in registers since the last iteration) goes to the other buffer, then its
-      // registers and this chunk's weight registers are refilled two chunks ahead
-      const int buf = (c - c_begin) & 1;
-      store_x(buf ^ 1, c + 1);  // past this split's last chunk it fills the buffer nobody reads
-      load_x(c + 2);
-      const bf16_t* xb = &Xs[buf][fr * SK_LDS_STRIDE + fk];
+      store_x(set ^ 1, set ^ 1, c + 1);  // past this split's last chunk it fills the buffer nobody reads
+      load_x(set ^ 1, c + 3);
+      const bf16_t* xb = &Xs[set][fr * SK_LDS_STRIDE + fk];
       u32x4 wcur[KS];
 #pragma unroll
       for (int s = 0; s < KS; ++s) wcur[s] = wr[set][s];
@@ -637,13 +641,13 @@ static int launch_splitk_reduce(const float* workspace, const float* bias, const
 }
 
 // Into how many k ranges the stream kernel splits K: an estimate in microseconds, fitted to measurements on MI355X
-// of weights from 5 MB to 130 MB at 32 and 64 rows.
-//   The workgroups (column tiles x ranges) go over the 256 CUs in rounds; a round costs about 2 us of its own plus
-//     its share of the time to stream the weights at 4.5 TB/s. With 192 column tiles 3 ranges give 576 workgroups:
-//     a quarter of the CUs takes three, the rest two, and the kernel lasts as long as with 2 ranges; 4 ranges give
-//     three to every CU.
-//   Weights of more than 6 us with fewer than two workgroups per CU: the loads in flight do not cover the memory
-//     latency (x 1.5).
+// of weights from 5 MB to 130 MB at 32 to 128 rows.
+//   Up to four workgroups (column tiles x ranges) stay on a CU at once. The slowest CU has r = ceil(workgroups / 256)
+//     of them and takes r times a workgroup's share of the time to stream the weights at 4.5 TB/s, plus about a
+//     microsecond each. With 192 column tiles 3 ranges give 576 workgroups: a quarter of the CUs takes three, the
+//     rest two, and the kernel lasts as long as with 2 ranges; 4 ranges give three to every CU.
+//   One workgroup on a CU does not have enough loads in flight to cover the memory latency (x 1.45), two nearly
+//     (x 1.12), three do: three per CU is the best shape where the partial sums allow it.
 //   More than one range: the second kernel's launch (3 us) and the partial sums, M x N floats per range that are
 //     written and read again (4 S M / K of the weights' bytes, mostly out of the caches: weighted half).
 static int stream_splits(int M, int N, int K) {
@@ -654,8 +658,9 @@ static int stream_splits(int M, int N, int K) {
   double best_cost = 1e30;
   for (int s = 1; s <= s_max; ++s) {
     const long wgs = (long)tiles * s;
-    double cost = (double)((wgs + 255) / 256) * (2.0 + t_stream * 256.0 / wgs);
-    if (wgs < 512 && t_stream > 6.0) cost *= 1.5;
+    const long r = (wgs + 255) / 256;
+    const double latency = r == 1 ? 1.45 : (r == 2 ? 1.12 : 1.0);
+    double cost = (double)r * (1.0 + t_stream * 256.0 / wgs * latency);
     if (s > 1) cost += 3.0 + 2.0 * s * M / K * t_stream;
     if (cost < best_cost - 1e-9) {
       best_cost = cost;
