@@ -554,18 +554,22 @@ gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
       store_x(set ^ 1, set ^ 1, c + 1);  // past this split's last chunk it fills the buffer nobody reads
       load_x(set ^ 1, c + 3);
       const bf16_t* xb = &Xs[set][fr * SK_LDS_STRIDE + fk];
-      u32x4 wcur[KS];
-#pragma unroll
-      for (int s = 0; s < KS; ++s) wcur[s] = wr[set][s];
-      load_w(set, c + 2);
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
           const u32x4 af = *reinterpret_cast<const u32x4*>(xb + t * 16 * SK_LDS_STRIDE + s * 32);
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(wcur[s]), acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(af), as_bf16x8(wr[set][s]), acc[t], 0, 0, 0);
         }
+      // the weight registers are refilled behind the products that read them: refilled ahead of them (from a copy),
+      // the new values landed in other registers and were moved into place at the end of the loop, which waits for
+      // loads issued a moment before
+      load_w(set, c + 2);
       lds_barrier();
+      // Nothing moves across the end of a chunk: the compiler had lifted the next chunk's masking of its a registers
+      // (a select per register) to the top of the loop, where it waited for every load in flight, the weights
+      // requested a moment before among them, and each pair of chunks cost a whole memory latency.
+      __builtin_amdgcn_sched_barrier(0);
     };
     int c = c_begin;
     for (; c + 1 < c_end; c += 2) {
