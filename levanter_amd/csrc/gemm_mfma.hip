@@ -606,10 +606,30 @@ splitk_reduce_kernel(const float* __restrict__ partial, const float* __restrict_
   if (idx >= total) return;
   const int m = (int)(idx / N), n = (int)(idx % N);
   if (VEC) {
-    f32x4 v = *reinterpret_cast<const f32x4*>(partial + idx);
-    for (int s = 1; s < S; ++s) {
-      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (size_t)s * total + idx);
-      v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+    // four ranges are requested at once and added in their order: a loop of load - add - load paid the latency of
+    // every range in turn (the partial sums come from other CUs, out of L2 at best)
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* src = partial + idx;
+    int s = 0;
+    for (; s + 4 <= S; s += 4) {
+      f32x4 p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p[j] = *reinterpret_cast<const f32x4*>(src + (size_t)(s + j) * total);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[0] += p[j][0]; v[1] += p[j][1]; v[2] += p[j][2]; v[3] += p[j][3];
+      }
+    }
+    {
+      f32x4 p[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j)  // the last ranges, unconditionally from a valid place
+        p[j] = *reinterpret_cast<const f32x4*>(src + (size_t)min(s + j, S - 1) * total);
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        if (s + j < S) {
+          v[0] += p[j][0]; v[1] += p[j][1]; v[2] += p[j][2]; v[3] += p[j][3];
+        }
     }
     float o[4] = {v[0], v[1], v[2], v[3]};
     if (bias) {
