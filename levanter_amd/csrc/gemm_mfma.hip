@@ -4,9 +4,9 @@
 //   tile kernel   (M > 128): a 256x256, 256x192, 256x128, 128x128 or 128x64 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 (K split into ranges, with a second kernel for the sums, where the tiles alone would leave CUs idle)
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
-//   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS, the weights go
-//                 straight into MFMA operand registers, K is split over workgroups and a second kernel
-//                 adds the partial sums in a fixed order;
+//   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
+//                 workgroup, the weights go straight into MFMA operand registers, K is split over workgroups
+//                 and a second kernel adds the partial sums in a fixed order;
 //   skinny kernel (M <= 24): a workgroup owns 16 output columns; its waves split K, load their part of w
 //                 straight into MFMA operand registers (16x16x32), and their partial sums are added
 //                 through LDS in a fixed order.
@@ -472,24 +472,26 @@ static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const floa
 // ------------------------------------------------------------------------------------------------
 // Stream kernel, for 24 < M <= 128: the weights are still the traffic that matters, but fetching the `a`
 // fragments from L2 once per wave (as the skinny kernel does) would cost more than the weights. Here a
-// workgroup of 4 waves owns 64 output columns (16 per wave) and all M rows; `a` goes through LDS in chunks of
-// 256 k and is shared by the 4 waves, each wave loads its own 16 weight rows straight into MFMA operand
+// workgroup of NW waves (4, 8, 12 or 16) owns NW x 16 output columns and all M rows; `a` goes through LDS in chunks
+// of 64 k and is shared by the waves, each wave loads its own 16 weight rows straight into MFMA operand
 // registers. To fill the chip the K range is split over `S` workgroups (blockIdx.y); with S > 1 the partial
 // sums go to a float32 workspace [S][M][N] and a second kernel adds them in order and applies the epilogue.
 #define SK_CHUNK 64
 #define SK_LDS_STRIDE (SK_CHUNK + 8)
 
-template <typename TO, int MT>
-__global__ void __launch_bounds__(256)
+template <typename TO, int MT, int NW>
+__global__ void __launch_bounds__(NW * 64)
 gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, float* __restrict__ partial, int M, int N, int K, int act,
                    int S) {
   constexpr int BM = MT * 16;
-  constexpr int XCH = BM * (SK_CHUNK / 8) / 256;  // 16-byte chunks of the a tile per thread (MT = 2: 2, 4: 4, 8: 8)
+  constexpr int NT = NW * 64;
+  constexpr int A_CHUNKS = BM * (SK_CHUNK / 8);       // 16-byte chunks of the a tile
+  constexpr int XCH = (A_CHUNKS + NT - 1) / NT;       // per thread (threads beyond the tile repeat its last chunk)
   __shared__ __attribute__((aligned(16))) bf16_t Xs[2][BM * SK_LDS_STRIDE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 15, fk = (lane >> 4) * 8;
-  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int n0 = blockIdx.x * (NW * 16) + wave * 16;
   const int split = blockIdx.y;
   const int n_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
   const int per = (n_chunks + S - 1) / S;
@@ -501,7 +503,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   int xk[XCH], xlds[XCH];
 #pragma unroll
   for (int i = 0; i < XCH; ++i) {
-    const int c = tid + 256 * i;
+    const int c = min(tid + NT * i, A_CHUNKS - 1);
     const int row = c / (SK_CHUNK / 8);
     xk[i] = (c % (SK_CHUNK / 8)) * 8;
     xoff[i] = (uint32_t)((size_t)min(row, M - 1) * lda);
@@ -664,31 +666,49 @@ static int launch_splitk_reduce(const float* workspace, const float* bias, const
   return lev_check_launch("linear_reduce");
 }
 
-// Into how many k ranges the stream kernel splits K: an estimate in microseconds, fitted to measurements on MI355X
-// of weights from 5 MB to 130 MB at 32 to 128 rows.
-//   Up to four workgroups (column tiles x ranges) stay on a CU at once. The slowest CU has r = ceil(workgroups / 256)
-//     of them and takes r times a workgroup's share of the time to stream the weights at 4.5 TB/s, plus about a
-//     microsecond each. With 192 column tiles 3 ranges give 576 workgroups: a quarter of the CUs takes three, the
-//     rest two, and the kernel lasts as long as with 2 ranges; 4 ranges give three to every CU.
-//   One workgroup on a CU does not have enough loads in flight to cover the memory latency (x 1.45), two nearly
-//     (x 1.12), three do: three per CU is the best shape where the partial sums allow it.
+// The shape of the stream kernel's launch: how many waves a workgroup has (16 columns each) and into how many k ranges
+// K is split. An estimate in microseconds of every combination, fitted to measurements on MI355X of weights from
+// 5 MB to 400 MB at 32 to 128 rows.
+//   What the CUs fetch is the weights once and the activations once per column tile: a wider workgroup shares its a
+//     tile among more columns (at 64 rows and 64 columns the a tiles are as many bytes as the weights). Together
+//     the CUs get about 7.5 TB/s out of L2.
+//   A CU holds 16 waves of this kernel. The slowest CU has r = ceil(workgroups / 256) workgroups and takes r times a
+//     workgroup's share of that time, plus about a microsecond each. With 4 or 8 waves on a CU the loads in flight do
+//     not cover the memory latency (x 1.45, x 1.12); 12 or 16 do.
 //   More than one range: the second kernel's launch (3 us) and the partial sums, M x N floats per range that are
 //     written and read again (4 S M / K of the weights' bytes, mostly out of the caches: weighted half).
-static int stream_splits(int M, int N, int K) {
-  const int tiles = (N + 63) / 64, chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+//   Measured at the 7B sizes, 64 rows (qkv / proj / fc / mproj, second kernel included): 4 waves 33 / 18 / 42 / 43 us,
+//     the shapes chosen here (12 x 4 ranges, 12 x 11, 16 x 4, 16 x 16) 29 / 17 / 40 / 38 us; at 128 rows 47 / 20 / 58 / 55
+//     against 37 / 22 / 46 / 45 us.
+struct StreamPlan {
+  int waves;   // waves of a workgroup (16 columns each): 4, 8, 12 or 16
+  int splits;  // k ranges
+};
+static StreamPlan plan_stream(int M, int N, int K) {
+  static const int nw[4] = {4, 8, 12, 16};
+  const int chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
   const int s_max = chunks / 2 < 16 ? (chunks / 2 < 1 ? 1 : chunks / 2) : 16;  // at least two chunks each
-  const double t_stream = (double)N * K * 2.0 / 4.5e6;
-  int best = 1;
+  const double w_bytes = (double)N * K * 2.0;
+  StreamPlan best = {4, 1};
   double best_cost = 1e30;
-  for (int s = 1; s <= s_max; ++s) {
-    const long wgs = (long)tiles * s;
-    const long r = (wgs + 255) / 256;
-    const double latency = r == 1 ? 1.45 : (r == 2 ? 1.12 : 1.0);
-    double cost = (double)r * (1.0 + t_stream * 256.0 / wgs * latency);
-    if (s > 1) cost += 3.0 + 2.0 * s * M / K * t_stream;
-    if (cost < best_cost - 1e-9) {
-      best_cost = cost;
-      best = s;
+  const int n_widths = w_bytes < 24e6 ? 1 : 4;  // weights of a few MB: the narrow workgroup measured best throughout
+  for (int i = 0; i < n_widths; ++i) {
+    const int tiles = (N + nw[i] * 16 - 1) / (nw[i] * 16);
+    const int per_cu = 16 / nw[i];  // workgroups that stay on a CU at once
+    const double a_bytes = (double)tiles * M * K * 2.0;  // every column tile reads all of a, once over its ranges
+    for (int s = 1; s <= s_max; ++s) {
+      const long wgs = (long)tiles * s;
+      const long r = (wgs + 255) / 256;  // workgroups of the slowest CU
+      if (r > per_cu && wgs > 256L * per_cu) continue;
+      const int waves_cu = (int)r * nw[i];
+      const double latency = waves_cu <= 4 ? 1.45 : (waves_cu <= 8 ? 1.12 : 1.0);
+      const double t = (w_bytes + a_bytes) / 7.5e6;  // microseconds at what the CUs get out of L2 together
+      double cost = (double)r * (1.0 + t * 256.0 / wgs * latency);
+      if (s > 1) cost += 3.0 + 2.0 * s * M / K * (w_bytes / 4.5e6);
+      if (cost < best_cost - 1e-9) {
+        best_cost = cost;
+        best = {nw[i], s};
+      }
     }
   }
   return best;
@@ -739,7 +759,7 @@ static TilePlan plan_tiles(int M, int N, int K) {
 
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
   if (M <= SKINNY_MAX_M) return 0;
-  const int S = M <= 128 ? stream_splits(M, N, K) : plan_tiles(M, N, K).splits;
+  const int S = M <= 128 ? plan_stream(M, N, K).splits : plan_tiles(M, N, K).splits;
   return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
 }
 
@@ -747,16 +767,28 @@ template <typename TO>
 static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
                          long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
   if ((size_t)M * lda >= (1ull << 32)) return lev_fail("linear: the activation matrix is too large (M=%d lda=%ld)", M, lda);
-  const int tiles = (N + 63) / 64;
-  const int S = stream_splits(M, N, K);
+  const StreamPlan plan = plan_stream(M, N, K);
+  const int S = plan.splits;
   if (S > 1 && !workspace) return lev_fail("linear: M=%d N=%d K=%d needs a workspace of lev_linear_mfma_workspace bytes", M, N, K);
-  dim3 grid(tiles, S);
-  if (M <= 32)
-    gemm_stream_kernel<TO, 2><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
-  else if (M <= 64)
-    gemm_stream_kernel<TO, 4><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
-  else
-    gemm_stream_kernel<TO, 8><<<grid, 256, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S);
+  dim3 grid((N + plan.waves * 16 - 1) / (plan.waves * 16), S);
+#define LEV_STREAM(MT_, NW_) \
+  gemm_stream_kernel<TO, MT_, NW_><<<grid, NW_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, S)
+#define LEV_STREAM_MT(MT_)                 \
+  switch (plan.waves) {                    \
+    case 4: LEV_STREAM(MT_, 4); break;     \
+    case 8: LEV_STREAM(MT_, 8); break;     \
+    case 12: LEV_STREAM(MT_, 12); break;   \
+    default: LEV_STREAM(MT_, 16); break;   \
+  }
+  if (M <= 32) {
+    LEV_STREAM_MT(2)
+  } else if (M <= 64) {
+    LEV_STREAM_MT(4)
+  } else {
+    LEV_STREAM_MT(8)
+  }
+#undef LEV_STREAM_MT
+#undef LEV_STREAM
   if (int rc = lev_check_launch("linear_stream")) return rc;
   if (S > 1) return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
   return 0;
