@@ -170,6 +170,36 @@ def test_linear_bf16_random_shapes_strides_and_epilogues(K):
         assert err < tol, (M, K_, N, lda, act, with_res, with_bias, out.dtype, err)
 
 
+@pytest.mark.parametrize("M,K_,N", [(64, 4096, 4096), (33, 4096, 3208), (100, 2048, 6151), (128, 8192, 1608), (48, 16384, 1000),
+                                    (26, 4096, 12288), (64, 1024, 50257)])
+def test_linear_bf16_large_weights_at_25_to_128_rows(K, M, K_, N):
+    """Weights of 24 MB and more at 25 to 128 rows: the stream kernel's workgroups of 8, 12 and 16 waves that share one
+    activation tile, with every epilogue, both output types, a row stride above K and a width that is no multiple
+    of 16, against the float64 statement."""
+    lda = K_ + 8
+    a = _rand(M, lda, dtype=torch.bfloat16, seed=M).to(DEV)[:, :K_]
+    w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=N).to(DEV)
+    bias = _rand(N, seed=3).to(DEV)
+    base = a.double() @ w.double().t()
+    # float32 output with bias and residual (in place)
+    out = _rand(M, N, seed=4).to(DEV)
+    want = base + bias.double() + out.double()
+    K.linear(a, w, bias, out, residual=out)
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-3
+    # bfloat16 output with bias and the tanh GELU
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    want = torch.nn.functional.gelu(base + bias.double(), approximate="tanh")
+    K.linear(a, w, bias, out, activation="gelu_new")
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-2
+    # plain, one large term among small ones: every column finds it
+    a2 = (a * 0.01).contiguous()
+    a2[:, K_ - 3] = 8.0
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.float32)
+    K.linear(a2, w, None, out)
+    want = a2.double() @ w.double().t()
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_strided_input_and_all_activations(K, dtype):
     M, K_, N = 9, 96, 40
