@@ -341,7 +341,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 // place of the k range, so that they do not all read the same part of `a` and the same residue of the weight
 // rows at the same time; the order of the sum depends on the column tile only, never on M or the batch.
 #define SKINNY_SLOTS 72  // 16-byte slots of one staged instruction: 8 rows x (8 chunks + 1 of padding)
-#define SKINNY_MAX_M 24  // measured: with two row tiles it beats the stream kernel up to here, at 32 rows no longer
+#define SKINNY_MAX_M 24  // with two row tiles; which of these row counts it takes: use_skinny()
 
 template <typename TO, int WAVES, int U, int ROT, int MT>
 __global__ void __launch_bounds__(WAVES * 64)
@@ -757,8 +757,17 @@ static TilePlan plan_tiles(int M, int N, int K) {
   return best;
 }
 
+// Which kernel takes M rows: the skinny one up to 16 rows; from 17 to SKINNY_MAX_M rows (two row tiles that share the
+// weight loads) except for large weights at 20 rows and more, where the stream kernel's shared activation tile wins
+// (measured at the 7B sizes, 24 rows: 100 MB weight 30 us against 26, 134 MB 38 against 35; 33 MB 13.5 against 16).
+static bool use_skinny(int M, int N, int K) {
+  if (M <= 16) return true;
+  if (M > SKINNY_MAX_M) return false;
+  return !(M >= 20 && (double)N * K * 2.0 >= 64e6);
+}
+
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
-  if (M <= SKINNY_MAX_M) return 0;
+  if (use_skinny(M, N, K)) return 0;
   const int S = M <= 128 ? plan_stream(M, N, K).splits : plan_tiles(M, N, K).splits;
   return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
 }
@@ -797,7 +806,7 @@ static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float
 template <typename TO>
 static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                              TO* out, long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
-  if (M <= SKINNY_MAX_M) {
+  if (use_skinny(M, N, K)) {
     launch_skinny<TO>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
   } else if (M <= 128) {
     return launch_stream<TO>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, stream);

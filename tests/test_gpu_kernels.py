@@ -171,9 +171,9 @@ def test_linear_bf16_random_shapes_strides_and_epilogues(K):
 
 
 @pytest.mark.parametrize("M,K_,N", [(64, 4096, 4096), (33, 4096, 3208), (100, 2048, 6151), (128, 8192, 1608), (48, 16384, 1000),
-                                    (26, 4096, 12288), (64, 1024, 50257), (128, 4096, 16384), (32, 4096, 16384)])
-def test_linear_bf16_large_weights_at_25_to_128_rows(K, M, K_, N):
-    """Weights of 24 MB and more at 25 to 128 rows: the stream kernel's workgroups of 8, 12 and 16 waves that share one
+                                    (26, 4096, 12288), (64, 1024, 50257), (128, 4096, 16384), (32, 4096, 16384), (22, 4096, 8200)])
+def test_linear_bf16_large_weights_at_20_to_128_rows(K, M, K_, N):
+    """Weights of 24 MB and more at 25 to 128 rows (64 MB and more from 20 rows): the stream kernel's workgroups of 8, 12 and 16 waves that share one
     activation tile, with every epilogue, both output types, a row stride above K and a width that is no multiple
     of 16, against the float64 statement."""
     lda = K_ + 8
