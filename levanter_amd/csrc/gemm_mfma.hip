@@ -4,7 +4,7 @@
 //   tile kernel   (M > 128): a 256x256, 256x192, 256x128, 128x128 or 128x64 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 (K split into ranges, with a second kernel for the sums, where the tiles alone would leave CUs idle)
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
-//   stream kernel (24 < M <= 128): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
+//   stream kernel (24 < M <= 128, large weights from 20 rows): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
 //                 workgroup, the weights go straight into MFMA operand registers, K is split over workgroups
 //                 and a second kernel adds the partial sums in a fixed order;
 //   skinny kernel (M <= 24): a workgroup owns 16 output columns; its waves split K, load their part of w
