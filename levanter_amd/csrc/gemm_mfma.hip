@@ -329,7 +329,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns 16 output columns; its WAVES
+// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns NT = 1 or 2 units of 16 output columns; its WAVES
 // waves split K. A wave takes pairs of adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
 //   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
 //   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
@@ -343,19 +343,25 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 #define SKINNY_SLOTS 72  // 16-byte slots of one staged instruction: 8 rows x (8 chunks + 1 of padding)
 #define SKINNY_MAX_M 24  // with two row tiles; which of these row counts it takes: use_skinny()
 
-template <typename TO, int WAVES, int U, int ROT, int MT>
+template <typename TO, int WAVES, int U, int ROT, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
+  static_assert(NT == 1 || NT == 2, "one or two column units per workgroup");
   constexpr int AI = 2 * MT;  // `a` instructions per pair of k-steps: 8 rows each
-  __shared__ f32x4 red[WAVES][MT][64];
+  __shared__ f32x4 red[WAVES][NT][MT][64];
   __shared__ u32x4 stage[WAVES][AI][SKINNY_SLOTS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int fr = lane & 15, kg = lane >> 4;
-  const bool n_ok = n0 + fr < N;
-  const bf16_t* wrow = w + (size_t)(n_ok ? n0 + fr : 0) * K + kg * 8;
+  bool n_ok[NT];
+  const bf16_t* wrow[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    n_ok[j] = n0 + 16 * j + fr < N;
+    wrow[j] = w + (size_t)(n_ok[j] ? n0 + 16 * j + fr : 0) * K + kg * 8;
+  }
   const int ar = lane >> 3, ac = lane & 7;  // `a` loads: row (0..7, instruction i adds 8 i) and chunk of the line
   bool a_ok[AI];
   const bf16_t* arow[AI];
@@ -372,30 +378,33 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
   // (which no other workgroup's streaming overlaps: all of them finish together) has no dependent loads left.
   // Unconditional loads from addresses that are always valid (clamped; `w` stands in for a missing operand):
   // a load under a condition would make the compiler wait for it at the join, ahead of the whole k loop.
-  float pre_bias;
-  f32x4 pre_res[MT];
-  {
-    const int nn = min(n0 + fr, N - 1);
+  float pre_bias[NT];
+  f32x4 pre_res[NT][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int nn = min(n0 + 16 * j + fr, N - 1);
     const float* bp = bias ? bias + nn : reinterpret_cast<const float*>(w);
-    pre_bias = *bp;
-    if (!bias) pre_bias = 0.f;
+    pre_bias[j] = *bp;
+    if (!bias) pre_bias[j] = 0.f;
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int m = min(t * 16 + kg * 4 + r, M - 1);
         const float* rp = residual ? residual + (size_t)m * ldr + nn : reinterpret_cast<const float*>(w);
-        pre_res[t][r] = *rp;
+        pre_res[j][t][r] = *rp;
       }
   }
 
-  f32x4 acc[MT];
+  f32x4 acc[NT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int npairs = (K + 63) / 64;
   const int rot = ROT ? (int)((blockIdx.x * 2654435761u) % (unsigned)npairs) : 0;
   for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
-    u32x4 wv[U][2], av[U][AI];
+    u32x4 wv[U][NT][2], av[U][AI];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int pr = p0 + u * WAVES;
@@ -405,9 +414,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
         pr = pr >= npairs ? pr - npairs : pr;
       }
       const int k = pr * 64;
-      const bool w_ok = p_ok && n_ok;
-      wv[u][0] = (w_ok && k + kg * 8 < K) ? load16(wrow + k) : u32x4{0, 0, 0, 0};
-      wv[u][1] = (w_ok && k + 32 + kg * 8 < K) ? load16(wrow + k + 32) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const bool w_ok = p_ok && n_ok[j];
+        wv[u][j][0] = (w_ok && k + kg * 8 < K) ? load16(wrow[j] + k) : u32x4{0, 0, 0, 0};
+        wv[u][j][1] = (w_ok && k + 32 + kg * 8 < K) ? load16(wrow[j] + k + 32) : u32x4{0, 0, 0, 0};
+      }
       const bool c_ok = p_ok && k + ac * 8 < K;
 #pragma unroll
       for (int i = 0; i < AI; ++i) av[u][i] = (c_ok && a_ok[i]) ? load16(arow[i] + k) : u32x4{0, 0, 0, 0};
@@ -420,23 +432,29 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const u32x4 a_lo = my_stage[2 * t * SKINNY_SLOTS + ld_slot], a_hi = my_stage[2 * t * SKINNY_SLOTS + ld_slot + 4];
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][0]), acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(wv[u][1]), acc[t], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][j][0]), acc[j][t], 0, 0, 0);
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(wv[u][j][1]), acc[j][t], 0, 0, 0);
+        }
       }
     }
   }
 #pragma unroll
-  for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) red[wave][j][t][lane] = acc[j][t];
   __syncthreads();
   // 16x16 accumulator: register r of lane l is row 4*(l/16) + r, column l%16. Partial sums are added in wave order.
-  if (wave == 0) {
-    const int nn = n0 + fr;
+  if (wave < NT) {  // wave j finishes column unit j
+    const int j = wave;
+    const int nn = n0 + 16 * j + fr;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      f32x4 s = red[0][t][lane];
+      f32x4 s = red[0][j][t][lane];
 #pragma unroll
       for (int v = 1; v < WAVES; ++v) {
-        const f32x4 o = red[v][t][lane];
+        const f32x4 o = red[v][j][t][lane];
         s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
       }
       if (nn < N) {
@@ -444,8 +462,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
         for (int r = 0; r < 4; ++r) {
           const int m = t * 16 + kg * 4 + r;
           if (m >= M) continue;
-          float v = lev_activate(s[r] + pre_bias, act);
-          if (residual) v += pre_res[t][r];
+          float v = lev_activate(s[r] + (j == 0 ? pre_bias[0] : pre_bias[NT - 1]), act);
+          if (residual) v += (j == 0 ? pre_res[0][t][r] : pre_res[NT - 1][t][r]);
           out[(size_t)m * ldo + nn] = from_float<TO>(v);
         }
       }
@@ -456,15 +474,24 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 // Choices measured on MI355X at K = 4096 .. 16384 and M = 1 .. 16 (graph replays over distinct weights): with many
 // column tiles 4 waves with 4 or 2 pairs in flight; with fewer than 512 the chip is only filled by 16 waves per
 // workgroup. The rotated start never costs and takes a third off the time where rows are long (K = 16384).
+// Two column units per workgroup (32 columns: every `a` fragment feeds two weight fragments, half the activation
+// traffic) pay where the halved number of workgroups still fills the chip evenly or the rows are many: 16384
+// columns x 4096 at 8 rows 28.1 -> 26.2 us, at 16 rows 33.4 -> 27.8 us; 24576 x 6144 at 16 rows 76 -> 64 us; at one
+// row and with workgroup counts that are no multiple of the CUs (18432 or 50257 columns) they lose up to 15 %.
 template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
   const int tiles = (N + 15) / 16;
-#define LEV_SKINNY(W_, U_, MT_) gemm_skinny_kernel<TO, W_, U_, 1, MT_><<<tiles, W_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act)
+#define LEV_SKINNY(W_, U_, MT_, NT_) \
+  gemm_skinny_kernel<TO, W_, U_, 1, MT_, NT_><<<(tiles + NT_ - 1) / NT_, W_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act)
   if (M <= 16) {
-    if (tiles >= 1024) LEV_SKINNY(4, 4, 1); else if (tiles >= 512) LEV_SKINNY(4, 2, 1); else LEV_SKINNY(16, 1, 1);
+    const bool two_units = tiles >= 1024 && (M >= 12 || (tiles / 2) % 256 == 0);
+    if (two_units) LEV_SKINNY(4, 2, 1, 2);
+    else if (tiles >= 1024) LEV_SKINNY(4, 4, 1, 1);
+    else if (tiles >= 512) LEV_SKINNY(4, 2, 1, 1);
+    else LEV_SKINNY(16, 1, 1, 1);
   } else {  // 17 .. SKINNY_MAX_M rows: two row tiles share every weight load
-    if (tiles >= 1024) LEV_SKINNY(4, 2, 2); else if (tiles >= 512) LEV_SKINNY(4, 2, 2); else LEV_SKINNY(16, 1, 2);
+    if (tiles >= 512) LEV_SKINNY(4, 2, 2, 1); else LEV_SKINNY(16, 1, 2, 1);
   }
 #undef LEV_SKINNY
 }
