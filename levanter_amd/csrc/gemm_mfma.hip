@@ -329,7 +329,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns NT = 1 or 2 units of 16 output columns; its WAVES
+// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns NT = 1 to 3 units of 16 output columns; its WAVES
 // waves split K. A wave takes pairs of adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
 //   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
 //   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
@@ -347,7 +347,7 @@ template <typename TO, int WAVES, int U, int ROT, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, const float* __restrict__ bias,
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
-  static_assert(NT == 1 || NT == 2, "one or two column units per workgroup");
+  static_assert(NT >= 1 && NT <= WAVES, "wave j finishes column unit j");
   constexpr int AI = 2 * MT;  // `a` instructions per pair of k-steps: 8 rows each
   __shared__ f32x4 red[WAVES][NT][MT][64];
   __shared__ u32x4 stage[WAVES][AI][SKINNY_SLOTS];
@@ -462,8 +462,15 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
         for (int r = 0; r < 4; ++r) {
           const int m = t * 16 + kg * 4 + r;
           if (m >= M) continue;
-          float v = lev_activate(s[r] + (j == 0 ? pre_bias[0] : pre_bias[NT - 1]), act);
-          if (residual) v += (j == 0 ? pre_res[0][t][r] : pre_res[NT - 1][t][r]);
+          float pb = pre_bias[0], pr = pre_res[0][t][r];
+#pragma unroll
+          for (int j2 = 1; j2 < NT; ++j2)
+            if (j == j2) {
+              pb = pre_bias[j2];
+              pr = pre_res[j2][t][r];
+            }
+          float v = lev_activate(s[r] + pb, act);
+          if (residual) v += pr;
           out[(size_t)m * ldo + nn] = from_float<TO>(v);
         }
       }
@@ -478,6 +485,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 // traffic) pay where the halved number of workgroups still fills the chip evenly or the rows are many: 16384
 // columns x 4096 at 8 rows 28.1 -> 26.2 us, at 16 rows 33.4 -> 27.8 us; 24576 x 6144 at 16 rows 76 -> 64 us; at one
 // row and with workgroup counts that are no multiple of the CUs (18432 or 50257 columns) they lose up to 15 %.
+// Three units and 16 waves for 12288 columns x 4096: 25.1 -> 21.8 us at 16 rows, the same at 8 rows, 10 % slower at one.
 template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
@@ -487,6 +495,7 @@ static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const floa
   if (M <= 16) {
     const bool two_units = tiles >= 1024 && (M >= 12 || (tiles / 2) % 256 == 0);
     if (two_units) LEV_SKINNY(4, 2, 1, 2);
+    else if (M >= 12 && tiles >= 720 && tiles < 1024) LEV_SKINNY(16, 1, 1, 3);  // about 256 workgroups of 48 columns
     else if (tiles >= 1024) LEV_SKINNY(4, 4, 1, 1);
     else if (tiles >= 512) LEV_SKINNY(4, 2, 1, 1);
     else LEV_SKINNY(16, 1, 1, 1);

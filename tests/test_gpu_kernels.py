@@ -98,6 +98,7 @@ LINEAR_SHAPES = [(1, 64, 192), (2, 96, 320), (7, 320, 96), (16, 64, 1000), (9, 4
                  (17, 96, 50257 // 16), (24, 200, 8200), (21, 1096, 16400), (25, 96, 300), (64, 4096, 528), (65, 256, 257), (130, 96, 300), (300, 1600, 520),
                  (257, 64, 50257 // 8), (520, 72, 33000),
                  (13, 264, 50257), (16, 1096, 16400), (2, 72, 16384),  # 1,024 column units and more: two units per workgroup
+                 (12, 520, 12288), (15, 264, 11531),  # 720 to 1,023 units at 12 to 16 rows: three units per workgroup
                  (300, 72, 12288), (300, 1032, 22002), (2048, 64, 6144), (256, 6144, 96),
                  (200, 8200, 300), (320, 6400, 1600), (300, 1600, 520)]  # few tiles and a long K: K is split into ranges  # the last four take the 128x128, 256x256, 256x128 and 256x192 tiles
 
