@@ -62,7 +62,13 @@ def main() -> int:
     cfg = LmConfig.from_dict(raw)
     ps = 16
     max_batch = max(args.batch, 1 if args.no_points else 64)
-    ctx_end = args.prompt_len + args.warmup + args.steps + 1
+    # Requests whose prompts are done first decode beside the prompt portions of the others: `early` tokens at most
+    # before the timed steps begin. Nobody may end, and no page may be missing, before the last timed step.
+    early = (max_batch * args.prompt_len + 2047) // 2048 + 8
+    ctx_end = args.prompt_len + early + args.warmup + args.steps + 1
+    if ctx_end > cfg.n_positions:
+        print(f"bench.py: prompt {args.prompt_len} + {early + args.warmup + args.steps + 1} steps exceed n_positions {cfg.n_positions}")
+        return 2
     pages_per_seq = (max(ctx_end, 2048) + ps - 1) // ps
     ecfg = InferenceEngineConfig(max_pages=max_batch * ((ctx_end + ps - 1) // ps) + pages_per_seq, max_seqs=max_batch, page_size=ps,
                                  max_pages_per_seq=pages_per_seq, compute_dtype=args.dtype, max_prefill_size=2048,
@@ -85,7 +91,7 @@ def main() -> int:
     def decode_run(batch, steps, warmup, seed):
         """Prefill ``batch`` prompts, then time ``steps`` decode steps. Returns (seconds, mean context)."""
         engine.reset()
-        reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=warmup + steps + 8, temperature=0.0)
+        reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=early + warmup + steps + 8, temperature=0.0)
                 for i, p in enumerate(prompts(batch, args.prompt_len, seed))]
         seqs = engine.enqueue_requests(reqs)
         while any(s.n_cached < s.prompt_len for s in seqs) or any(not s.generated for s in seqs):
@@ -93,13 +99,13 @@ def main() -> int:
         for _ in range(warmup):
             engine.step()
         torch.cuda.synchronize()
-        ctx0 = seqs[0].n_cached
+        ctx0 = sum(s.n_cached for s in seqs) / len(seqs)
         t = time.perf_counter()
         for _ in range(steps):
             engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        assert all(len(s.generated) >= warmup + steps for s in seqs), "the timed steps did not all decode the whole batch"
+        assert all(len(s.generated) >= warmup + steps and not s.done for s in seqs), "the timed steps did not all decode the whole batch"
         ctx_mean = ctx0 + (steps + 1) / 2.0
         engine.reset()
         return dt, ctx_mean
