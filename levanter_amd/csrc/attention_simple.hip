@@ -5,7 +5,9 @@
 //   keys  [page][kv_head][HD/8][PS][8], values [page][kv_head][HD][PS]
 //   positions[t]: absolute position of query t; it sees keys at positions p with
 //                 max(0, pos - window + 1) <= p <= pos   (window 0: all)
-//   token_seq[t]: row of block_tables (page ids of that request, -1 where none)
+//   token_seq[t]: row of block_tables (page ids of that request, -1 where none). A key whose block has no page
+//                 is treated as masked and never loaded (a padding token of a replayed step may name a block that
+//                 its request has given back); a query with no key at all gives zeros.
 #include "common.h"
 
 #define AS_MAX_HD 512
@@ -34,11 +36,12 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
   const size_t head_elems = (size_t)HD * PS;
   for (int c0 = (first / 64) * 64; c0 <= pos; c0 += 64) {
     const int kp = c0 + lane;
-    const bool live = kp >= first && kp <= pos;
+    bool live = kp >= first && kp <= pos;
     float s = -INFINITY;
     int page = -1;
+    if (live) page = bt[kp / PS];
+    live = live && page >= 0;
     if (live) {
-      page = bt[kp / PS];
       const int off = kp % PS;
       const T* kb = k_pages + ((size_t)page * KVH + kvh) * head_elems;
       float dot = 0.f;
@@ -46,7 +49,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
       s = dot;
     }
     const float m_new = fmaxf(m, wave_max(s));
-    const float p = live ? expf(s - m_new) : 0.f;
+    const float p = live ? expf(s - m_new) : 0.f;  // no live key so far: m_new = -inf, p = 0
     const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
     l = l * corr + wave_sum(p);
     m = m_new;
@@ -71,7 +74,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
     }
     __syncthreads();
   }
-  const float inv = 1.0f / l;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int i = 0; i < ND; ++i) {
     const int d = lane + 64 * i;

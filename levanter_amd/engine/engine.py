@@ -44,7 +44,7 @@ class InferenceEngine:
         self.runner = ModelRunner(model, self.cache, env, allocate=allocate)
         self.sampler = Sampler(env.kernels, env.device)
         self.scheduler = Scheduler(self.cache, config, self.runner.max_len)
-        self.stats = {"steps": 0, "tokens_in": 0, "device_s": 0.0}
+        self.stats = {"steps": 0, "commits": 0, "tokens_in": 0, "device_s": 0.0}
         self._pending: Optional[_Launched] = None  # a step launched ahead of the one being committed
 
     # ---- construction -------------------------------------------------------------------------
@@ -125,6 +125,7 @@ class InferenceEngine:
             if not plan:
                 return []
             pend = self._launch(plan, None)
+        self.stats["commits"] += 1
         nxt = None
         if self.config.decode_lookahead:
             ahead = self.scheduler.plan_lookahead(pend.plan)
@@ -167,9 +168,11 @@ class InferenceEngine:
         t0 = time.perf_counter()
         idle_steps = 0
         while not all(s.done for s in seqs):
-            n_before = self.stats["steps"]
+            # progress: a step was launched, a step launched earlier was committed, or a sequence ended (the planner
+            # ends a lone sequence that the pool cannot hold without launching anything)
+            before = (self.stats["steps"], self.stats["commits"], sum(s.done for s in seqs))
             self.step()
-            idle_steps = idle_steps + 1 if self.stats["steps"] == n_before else 0
+            idle_steps = idle_steps + 1 if (self.stats["steps"], self.stats["commits"], sum(s.done for s in seqs)) == before else 0
             if idle_steps >= 2:  # the reference breaks after two iterations without progress (engine.py:1160-1171)
                 raise RuntimeError("the scheduler made no step twice in a row although requests are unfinished")
         dt = time.perf_counter() - t0

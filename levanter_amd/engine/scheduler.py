@@ -59,6 +59,8 @@ class Sequence_:
     done: bool = False
     finish_reason: str = ""
     n_preempted: int = 0
+    last_step: int = 0
+    """Number of the last planned step that held tokens of this sequence (who decodes next when a step cannot hold all)."""
 
     @property
     def n_cached(self) -> int:
@@ -86,6 +88,7 @@ class Scheduler:
         self.running: List[Sequence_] = []
         self._arrivals = 0
         self._steps_since_admission = 0
+        self._step_no = 0
         self.n_preemptions = 0
 
     # ---- intake -----------------------------------------------------------------------------
@@ -134,7 +137,7 @@ class Scheduler:
             entries, starved = self._pick()
             if not starved:
                 if entries:
-                    self._steps_since_admission += 1
+                    self._planned(entries)
                 return entries
             # pages ran out: preempt the youngest running sequence, or fail the only one
             victim = max(self.running, key=lambda s: s.order)
@@ -144,6 +147,19 @@ class Scheduler:
                     return []
                 continue
             self._preempt(victim)
+
+    def _planned(self, entries: List[PlannedEntry]) -> None:
+        self._steps_since_admission += 1
+        self._step_no += 1
+        for e in entries:
+            e.seq.last_step = self._step_no
+
+    @staticmethod
+    def _turn(seq: Sequence_):
+        """Who decodes first when ``max_tokens_per_round`` is below the number of decoding sequences: the one that
+        has waited longest, then the oldest. The reference's queue of pending tokens rotates the same way
+        (src/levanter/inference/jit_scheduler.py:524-577): what a round leaves over goes first in the next."""
+        return (seq.last_step, seq.order)
 
     def _taker(self):
         """take(seq, n): count the pages that n more tokens of seq need against what the pools have left."""
@@ -186,8 +202,8 @@ class Scheduler:
         entries: List[PlannedEntry] = []
         starved = False
         decoding = [s for s in self.running if s.n_cached >= s.prompt_len and s.n_pending == 1]
-        decoding.sort(key=lambda s: s.order)
-        for seq in decoding[: self.cfg.imputed_max_tokens_per_round]:
+        decoding.sort(key=self._turn)
+        for seq in sorted(decoding[: self.cfg.imputed_max_tokens_per_round], key=lambda s: s.order):
             if take(seq, 1):
                 entries.append(PlannedEntry(seq, [seq.tokens[-1]], True))
             else:
@@ -202,35 +218,37 @@ class Scheduler:
         entries come first). Prompt portions and admissions follow as in ``plan``, from what the host knows. Requests
         that end by length with ``pending``'s token are left out; one that ends by a stop sequence cannot be foreseen
         and is skipped when this step is committed (so are the pages and the slot it would have given back: the plan is
-        made as if nobody ended). Nothing is preempted here. None: wait for the tokens and plan as usual."""
+        made as if nobody ended). Sequences whose next token the host knows already (``max_tokens_per_round`` left them
+        out of ``pending``) stand behind the fed ones; who decodes is decided by turns as in ``plan``. Nothing is
+        preempted here. None: wait for the tokens and plan as usual."""
         if not pending or any(e.seq.done for e in pending):
             return None
         row_of: Dict[int, int] = {}
         for e in pending:
             if e.wants_logits:
                 row_of[id(e.seq)] = len(row_of)
-        # a request that decodes a token the host knows would have to stand among the fed ones
-        if any(s.n_cached >= s.prompt_len and s.n_pending == 1 for s in self.running):
-            return None
-        decoders = sorted((s for s in self.running if id(s) in row_of), key=lambda s: s.order)
-        if len(decoders) > self.cfg.imputed_max_tokens_per_round:
-            return None
+        fed = [s for s in self.running if id(s) in row_of
+               and len(s.tokens) + 1 < min(s.request.decode_params.max_num_tokens, self.max_len)]  # else pending's token is its last
+        known = [s for s in self.running if id(s) not in row_of and s.n_cached >= s.prompt_len and s.n_pending == 1]
+        chosen = sorted(fed + known, key=self._turn)[: self.cfg.imputed_max_tokens_per_round]
         if self._steps_since_admission >= self.cfg.max_rounds or any(s.n_cached < s.prompt_len for s in self.running):
             self._admit()
             self._steps_since_admission = 0
         take, free = self._taker()
         entries: List[PlannedEntry] = []
         rows: List[int] = []
-        for seq in decoders:
-            if len(seq.tokens) + 1 >= min(seq.request.decode_params.max_num_tokens, self.max_len):
-                continue  # pending's token is its last
+        for seq in sorted((s for s in chosen if id(s) in row_of), key=lambda s: s.order):
             if not take(seq, 1):
                 return None  # pages run out: the ordinary plan decides whom to preempt
             entries.append(PlannedEntry(seq, [0], True))
             rows.append(row_of[id(seq)])
+        for seq in sorted((s for s in chosen if id(s) not in row_of), key=lambda s: s.order):
+            if not take(seq, 1):
+                return None
+            entries.append(PlannedEntry(seq, [seq.tokens[-1]], True))
         if self._pick_portions(entries, take, free) or not entries:
             return None
-        self._steps_since_admission += 1
+        self._planned(entries)
         return entries, rows
 
     def _preempt(self, seq: Sequence_) -> None:

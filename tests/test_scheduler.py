@@ -263,3 +263,55 @@ def test_steps_with_prompt_portions_and_admissions_are_launched_ahead_too(seed):
     assert with_la == without
     assert none_ahead == 0 and ahead > 0
     assert any(max(b) > 1 and len(b) > 1 for b in batches_la)  # portions of prompts beside decoded tokens in one step
+
+
+@pytest.mark.parametrize("lookahead", [True, False])
+def test_a_lone_request_that_runs_out_of_pages_while_decoding_ends_with_its_own_error(lookahead):
+    # 2 pages of 16 tokens: a prompt of 10 tokens decodes until position 32 would need a third page
+    engine, _ = make_engine(DummyModel(vocab_size=50, count=True), max_pages=2, max_pages_per_seq=8, decode_lookahead=lookahead)
+    other = Request(prompt_tokens=[7], request_id=1, max_new_tokens=2)
+    res = engine.generate([Request(prompt_tokens=[1] * 10, request_id=0, max_new_tokens=40), other])
+    assert res.finish_reasons[0].startswith("error: out of pages")
+    # tokens 10 .. 31 are in the cache (22 generated ones were fed back) and the 23rd was sampled from the last step
+    assert res.tokens[0] == [(2 + i) % 50 for i in range(len(res.tokens[0]))] and len(res.tokens[0]) in (22, 23)
+    assert res.finish_reasons[1] == "length" and res.tokens[1] == [8, 9]  # the other request's result is not lost
+    assert all_released(engine)
+
+
+@pytest.mark.parametrize("lookahead", [True, False])
+def test_fewer_tokens_a_round_than_decoding_requests_take_turns(lookahead):
+    """``max_tokens_per_round`` below the number of decoding requests: nobody waits for the older ones to end."""
+    engine, model = make_engine(DummyModel(vocab_size=100, count=True), max_tokens_per_round=2, decode_lookahead=lookahead)
+    reqs = [Request(prompt_tokens=[10 * i + 1], request_id=i, max_new_tokens=6) for i in range(4)]
+    seqs = engine.enqueue_requests(reqs)
+    engine.step()  # the four prompts (one token each) in one step
+    progress = []
+    ahead = 0
+    while not all(s.done for s in seqs):
+        engine.step()
+        ahead += engine._pending is not None
+        progress.append([len(s.generated) for s in seqs])
+    for a, b in zip(progress, progress[2:]):  # within any two steps every unfinished request has advanced
+        assert all(y > x or y == 6 for x, y in zip(a, b)), (a, b)
+    assert all(len(b) <= 2 for b in model.batches[1:])
+    assert [s.generated for s in seqs] == [[10 * i + 2 + j for j in range(6)] for i in range(4)]
+    assert (ahead > 0) == lookahead  # steps are still launched ahead
+    assert all_released(engine)
+
+
+def test_max_rounds_is_the_number_of_decode_steps_between_two_looks_at_the_queue():
+    engine, model = make_engine(DummyModel(vocab_size=100, count=True), max_rounds=4, decode_lookahead=False)
+    first = engine.enqueue_requests([Request(prompt_tokens=[1, 2, 3], request_id=0, max_new_tokens=30)])
+    engine.step()
+    engine.step()
+    late = engine.enqueue_requests([Request(prompt_tokens=[50, 51], request_id=1, max_new_tokens=3)])
+    n0 = len(model.batches)
+    while not late[0].done:
+        engine.step()
+    joined = next(i for i, b in enumerate(model.batches) if len(b) == 2)
+    # the queue was looked at before step 0; steps 0 .. 3 run without a look, step 4 follows the next one
+    assert joined > n0 and joined == 4
+    assert model.batches[joined] == [1, 2]
+    assert late[0].generated == [52, 53, 54]
+    engine.reset()
+    assert all_released(engine)
