@@ -1,5 +1,6 @@
 // Embedding gather-add, LayerNorm / RMSNorm, the write of new keys and values into pages, sampling.
 #include "common.h"
+#include "sample_static.h"
 
 // ------------------------------------------------------------------------------------------
 // x[t, :] = float(table[token_t, :]) + float(pos_table[pos_t, :])        (32-bit residual stream)
@@ -417,4 +418,42 @@ extern "C" int lev_sample(const float* logits, long row_stride, const float* tem
   if (int rc = lev_check_launch("sample")) return rc;
   sample_merge_kernel<<<R, 64, 0, stream>>>(logits, row_stride, temperature, workspace, tokens, logprobs, V);
   return lev_check_launch("sample merge");
+}
+
+// ---- the same sampling from a scratch array of the library's own (see sample_static.h) -----------------------
+// In host code `sample_scratch` is only a stand-in for the symbol: the address a kernel can use comes from
+// hipGetSymbolAddress, once per device, and is kept in g_sample_scratch[device].
+#define LEV_MAX_DEVICES 64
+static __device__ __align__(256) float sample_scratch[(size_t)LEV_SAMPLE_STATIC_MAX_ROWS * SAMPLE_PARTS * 4];
+static float* g_sample_scratch[LEV_MAX_DEVICES];  // written once per device with one value: racing initialisers agree
+
+static int sample_scratch_ptr(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return lev_fail("sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= LEV_MAX_DEVICES) return lev_fail("sample_static: device %d is beyond the %d this library keeps scratch for", dev, LEV_MAX_DEVICES);
+  float* p = __atomic_load_n(&g_sample_scratch[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(sample_scratch));
+    if (e != hipSuccess || !p) return lev_fail("sample_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    __atomic_store_n(&g_sample_scratch[dev], p, __ATOMIC_RELEASE);
+  }
+  *out = p;
+  return 0;
+}
+
+extern "C" int lev_sample_static_init() {
+  float* p = nullptr;
+  return sample_scratch_ptr(&p);
+}
+
+extern "C" int lev_sample_static_max_rows() { return LEV_SAMPLE_STATIC_MAX_ROWS; }
+
+extern "C" int lev_sample_static(const float* logits, long row_stride, const float* temperature, const uint32_t* keys,
+                                 const int* positions, int* tokens, float* logprobs, int R, int V, hipStream_t stream) {
+  LEV_REQUIRE(R <= LEV_SAMPLE_STATIC_MAX_ROWS, "sample_static: %d rows are more than the %d its scratch array holds; use lev_sample with a workspace",
+              R, LEV_SAMPLE_STATIC_MAX_ROWS);
+  float* scratch = nullptr;
+  if (int rc = sample_scratch_ptr(&scratch)) return rc;
+  return lev_sample(logits, row_stride, temperature, keys, positions, tokens, logprobs, scratch, R, V, stream);
 }
