@@ -76,11 +76,29 @@ def find_hipcc() -> Optional[str]:
     return None
 
 
+def _with_includes(names: Iterable[str]) -> List[str]:
+    """The given sources and every file of ``csrc/`` that they include with ``#include "..."``, directly or not."""
+    seen, todo = set(), list(names)
+    while todo:
+        name = todo.pop()
+        if name in seen:
+            continue
+        seen.add(name)
+        with open(os.path.join(CSRC, name), encoding="utf-8") as f:
+            for line in f:
+                line = line.strip()
+                if line.startswith("#include \""):
+                    inc = line.split('"')[1]
+                    if os.path.isfile(os.path.join(CSRC, inc)):
+                        todo.append(inc)
+    return sorted(seen)
+
+
 def source_hash(unit: str = "core") -> str:
-    """Hash of what a unit is built from: the flags, its own sources and defines, and every header."""
+    """Hash of what a unit is built from: the flags, its own sources and defines, and the headers they include."""
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    names = sorted({src for src, _, _ in UNITS[unit]} | {n for n in os.listdir(CSRC) if n.endswith(".h")})
+    names = _with_includes(src for src, _, _ in UNITS[unit])
     for name in names:
         h.update(name.encode())
         with open(os.path.join(CSRC, name), "rb") as f:
