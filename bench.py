@@ -22,8 +22,11 @@ HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 
+GENERATED = 256  # the benchmark's requests generate this many tokens after their prompt
+
+
 def load_baseline_config():
-    """Layer sizes of BASELINE.json's configs[2] (the repo's gpt2_7b shape)."""
+    """Layer sizes of the reference's gpt2_7b configuration (config/gpt2_7b.yaml) with GPT-2's vocabulary."""
     return {"model_type": "gpt2", "n_layer": 32, "n_embd": 4096, "n_head": 32, "n_inner": 16384, "vocab_size": 50257,
             "n_positions": 2048, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
 
@@ -40,7 +43,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b"],
-                    help="decode: the contract above. xl_mix / 20b: the continuous-batching workloads of BASELINE.json's configs[3] / configs[4] "
+                    help="decode: the contract above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
                          "through InferenceEngine.generate; they print their own line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -65,9 +68,12 @@ def main() -> int:
     # Requests whose prompts are done first decode beside the prompt portions of the others: `early` tokens at most
     # before the timed steps begin. Nobody may end, and no page may be missing, before the last timed step.
     early = (max_batch * args.prompt_len + 2047) // 2048 + 8
-    ctx_end = args.prompt_len + early + args.warmup + args.steps + 1
+    # The timed steps lie in the middle of the GENERATED tokens that follow the prompt, however few they are: their mean
+    # context is prompt_len + GENERATED / 2 (untimed steps lead up to them).
+    span = max(args.steps, GENERATED)
+    ctx_end = args.prompt_len + early + args.warmup + span + 1
     if ctx_end > cfg.n_positions:
-        print(f"bench.py: prompt {args.prompt_len} + {early + args.warmup + args.steps + 1} steps exceed n_positions {cfg.n_positions}")
+        print(f"bench.py: prompt {args.prompt_len} + {early + args.warmup + span + 1} steps exceed n_positions {cfg.n_positions}")
         return 2
     pages_per_seq = (max(ctx_end, 2048) + ps - 1) // ps
     ecfg = InferenceEngineConfig(max_pages=max_batch * ((ctx_end + ps - 1) // ps) + pages_per_seq, max_seqs=max_batch, page_size=ps,
@@ -91,12 +97,15 @@ def main() -> int:
     def decode_run(batch, steps, warmup, seed):
         """Prefill ``batch`` prompts, then time ``steps`` decode steps. Returns (seconds, mean context)."""
         engine.reset()
-        reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=early + warmup + steps + 8, temperature=0.0)
+        reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=early + warmup + max(steps, GENERATED) + 8, temperature=0.0)
                 for i, p in enumerate(prompts(batch, args.prompt_len, seed))]
         seqs = engine.enqueue_requests(reqs)
         while any(s.n_cached < s.prompt_len for s in seqs) or any(not s.generated for s in seqs):
             engine.step()
         for _ in range(warmup):
+            engine.step()
+        ctx_now = sum(s.n_cached for s in seqs) / len(seqs)
+        for _ in range(max(0, int(args.prompt_len + GENERATED / 2.0 - (steps + 1) / 2.0 - ctx_now))):
             engine.step()
         torch.cuda.synchronize()
         ctx0 = sum(s.n_cached for s in seqs) / len(seqs)
@@ -140,8 +149,8 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
         "config": {"model": "gpt2_7b shape", "n_layer": L, "n_layer_full": full_layers, "n_embd": D, "n_head": cfg.n_head,
                    "head_dim": cfg.head_dim, "n_inner": F, "vocab_size": V, "n_positions": cfg.n_positions,
-                   "global_batch": args.batch, "seq_len": args.prompt_len + args.steps, "prompt_len": args.prompt_len,
-                   "page_size": ps, "parallelism": "single GPU"},
+                   "global_batch": args.batch, "seq_len": args.prompt_len + GENERATED, "prompt_len": args.prompt_len,
+                   "generated": GENERATED, "ctx_mean": round(ctx_mean, 1), "page_size": ps, "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
                      "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4)},
     }
@@ -186,19 +195,14 @@ def serving_workload(args) -> int:
     V = cfg.vocab_size
     pages_per_seq = (max(lens) + new_tokens + ps) // ps
     itemsize = 2 if args.dtype == "bfloat16" else 4
-    if args.workload == "20b":  # the cache takes what the weights leave of the memory (a margin for activations kept)
-        free, _total = torch.cuda.mem_get_info()
-        weights = 12 * cfg.n_layer * cfg.n_embd * cfg.n_embd * itemsize + V * cfg.n_embd * itemsize
-        page_bytes = 2 * cfg.n_layer * cfg.n_embd * itemsize * ps
-        max_pages = int(max(free - weights - (24 << 30), 0) // page_bytes)
-        max_pages = max(max_pages, n_req * pages_per_seq // 2)
-    else:
-        max_pages = n_req * pages_per_seq
-    ecfg = InferenceEngineConfig(max_pages=max_pages, max_seqs=n_req, page_size=ps, max_pages_per_seq=pages_per_seq,
+    # 20b: the engine sizes the cache itself from what the weights leave of the memory (at most every request at full length)
+    ecfg = InferenceEngineConfig(max_pages="auto" if args.workload == "20b" else n_req * pages_per_seq, cache_memory_reserve_gib=24.0,
+                                 max_seqs=n_req, page_size=ps, max_pages_per_seq=pages_per_seq,
                                  compute_dtype=args.dtype, max_prefill_size=chunk, max_seqs_in_prefill=n_req, seed=0)
     t0 = time.time()
     engine = InferenceEngine.from_config(cfg, seed=0, config=ecfg)
     torch.cuda.synchronize()
+    max_pages = engine.cache.groups[0].pool.n_pages
     print(f"[bench] model ready in {time.time() - t0:.1f}s: {engine.model.weight_bytes() / 1e9:.2f} GB of weights, "
           f"{max_pages} pages of {ps} tokens", file=sys.stderr, flush=True)
 

@@ -153,24 +153,35 @@ class SequenceHandle:
     closed: bool = False
 
 
+def group_units(requirements: Sequence[Tuple[int, object]]) -> Tuple[Dict[PagedKv, List[int]], Dict[int, SlotState]]:
+    """Sort (cache unit id, requirement) pairs: paged units by requirement (each distinct one is a group, in order of
+    first appearance), slot-state units by id."""
+    by_req: Dict[PagedKv, List[int]] = {}
+    slot_reqs: Dict[int, SlotState] = {}
+    for unit, req in requirements:
+        if isinstance(req, PagedKv):
+            by_req.setdefault(req, []).append(unit)
+        elif isinstance(req, SlotState):
+            slot_reqs[unit] = req
+        elif req is not None:
+            raise TypeError(f"cache unit {unit}: unknown cache requirement {req!r}")
+    return by_req, slot_reqs
+
+
 class CacheManager:
-    def __init__(self, requirements: Sequence[Tuple[int, object]], *, n_pages: int, page_size: int, max_seqs: int,
+    def __init__(self, requirements: Sequence[Tuple[int, object]], *, n_pages, page_size: int, max_seqs: int,
                  max_pages_per_seq: int):
-        """``requirements``: (cache unit id, PagedKv | SlotState | None) of every unit."""
+        """``requirements``: (cache unit id, PagedKv | SlotState | None) of every unit. ``n_pages``: pages of every
+        group's pool, or one number per group (in the order of ``group_units``)."""
         self.page_size = page_size
         self.max_seqs = max_seqs
         self.max_pages_per_seq = max_pages_per_seq
-        by_req: Dict[PagedKv, List[int]] = {}
-        slot_reqs: Dict[int, SlotState] = {}
-        for unit, req in requirements:
-            if isinstance(req, PagedKv):
-                by_req.setdefault(req, []).append(unit)
-            elif isinstance(req, SlotState):
-                slot_reqs[unit] = req
-            elif req is not None:
-                raise TypeError(f"cache unit {unit}: unknown cache requirement {req!r}")
+        by_req, slot_reqs = group_units(requirements)
+        counts = [int(n_pages)] * len(by_req) if isinstance(n_pages, (int, np.integer)) else [int(n) for n in n_pages]
+        if len(counts) != len(by_req):
+            raise ValueError(f"{len(counts)} page counts for {len(by_req)} cache groups")
         self.groups: List[PagedGroup] = [
-            PagedGroup(i, req, units, n_pages, page_size, max_seqs, max_pages_per_seq) for i, (req, units) in enumerate(by_req.items())
+            PagedGroup(i, req, units, counts[i], page_size, max_seqs, max_pages_per_seq) for i, (req, units) in enumerate(by_req.items())
         ]
         self.group_of_unit: Dict[int, PagedGroup] = {u: g for g in self.groups for u in g.units}
         self.state = StateSlots(slot_reqs, max_seqs)

@@ -7,15 +7,19 @@ GPU with a host-side scheduler; the differences are stated per field.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Union
 
 from .lm_config import ConfigError
 
 
 @dataclass(frozen=True)
 class InferenceEngineConfig:
-    max_pages: Optional[int] = None
-    """Pages in each cache group's pool. None: ``max_seqs * max_pages_per_seq`` (engine.py:108-111)."""
+    max_pages: Union[None, int, str] = None
+    """Pages in the pool of each cache group that keeps all keys (a group that keeps a window takes what it can use).
+    None: ``max_seqs * max_pages_per_seq`` (engine.py:108-111). "auto": what is free on the GPU once the weights are
+    loaded, less ``cache_memory_reserve_gib``, and at most ``max_seqs * max_pages_per_seq``. (Ours.)"""
+    cache_memory_reserve_gib: float = 8.0
+    """With ``max_pages="auto"``: device memory left alone for activations and kernel workspaces. (Ours.)"""
     max_seqs: int = 16
     """Most requests that are live (hold a slot) at a time (engine.py:66)."""
     page_size: int = 16
@@ -57,11 +61,19 @@ class InferenceEngineConfig:
         for name in ("max_seqs", "max_pages_per_seq", "max_seqs_in_prefill", "max_rounds"):
             if getattr(self, name) <= 0:
                 raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
-        if self.max_pages is not None and self.max_pages <= 0:
+        if isinstance(self.max_pages, str):
+            if self.max_pages != "auto":
+                raise ConfigError(f'max_pages must be a positive number, null or "auto", got {self.max_pages!r}')
+        elif self.max_pages is not None and self.max_pages <= 0:
             raise ConfigError(f"max_pages must be positive, got {self.max_pages}")
+        if self.cache_memory_reserve_gib < 0:
+            raise ConfigError(f"cache_memory_reserve_gib must not be negative, got {self.cache_memory_reserve_gib}")
 
     @property
     def imputed_max_pages(self) -> int:
+        """The page count of a group that keeps all keys, where it is known without asking the device."""
+        if self.max_pages == "auto":
+            raise ConfigError('max_pages="auto" is resolved when the cache is made, from the free device memory')
         return int(self.max_pages) if self.max_pages is not None else int(self.max_seqs * self.max_pages_per_seq)
 
     @property

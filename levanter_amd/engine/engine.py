@@ -40,7 +40,7 @@ class InferenceEngine:
         self.model = model
         self.config = config
         self.env = env
-        self.cache = make_cache(model, config)
+        self.cache = make_cache(model, config, env)
         self.runner = ModelRunner(model, self.cache, env, allocate=allocate)
         self.sampler = Sampler(env.kernels, env.device)
         self.scheduler = Scheduler(self.cache, config, self.runner.max_len)

@@ -9,7 +9,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from levanter_amd.cache import CacheManager
+from levanter_amd.cache import CacheManager, group_units, pages_per_group
 from levanter_amd.config import InferenceEngineConfig, LmConfig
 from levanter_amd.kernels import get_kernels
 from levanter_amd.parts import BuildEnv, DecoderLm
@@ -50,6 +50,24 @@ def random_model(config: LmConfig, seed: int, env: BuildEnv) -> DecoderLm:
     return DecoderLm(spec, tensors, env)
 
 
-def make_cache(model: DecoderLm, cfg: InferenceEngineConfig) -> CacheManager:
-    return CacheManager(model.cache_requirements(), n_pages=cfg.imputed_max_pages, page_size=cfg.page_size,
-                        max_seqs=cfg.max_seqs, max_pages_per_seq=cfg.max_pages_per_seq)
+def _free_device_bytes(device) -> int:
+    free, _total = torch.cuda.mem_get_info(device)
+    return int(free)
+
+
+def make_cache(model: DecoderLm, cfg: InferenceEngineConfig, env: Optional[BuildEnv] = None, free_bytes=None) -> CacheManager:
+    """The cache manager of a model under an engine configuration. Every cache group gets a pool of its own size:
+    ``max_pages`` (or ``max_seqs * max_pages_per_seq``) pages where all keys are kept, what the window and a step's
+    longest portion can touch where only a window is; with ``max_pages="auto"`` what is free on the device now (call
+    this once the weights are there) less ``cache_memory_reserve_gib``. ``free_bytes``: a stand-in for the query."""
+    requirements = model.cache_requirements()
+    by_req, _ = group_units(requirements)
+    if free_bytes is None and env is not None and env.device.type == "cuda":
+        free_bytes = lambda: _free_device_bytes(env.device)
+    itemsize = 4 if cfg.compute_dtype == "float32" else 2
+    counts = pages_per_group([(req, len(units)) for req, units in by_req.items()], max_pages=cfg.max_pages, page_size=cfg.page_size,
+                             max_seqs=cfg.max_seqs, max_pages_per_seq=cfg.max_pages_per_seq,
+                             longest_portion=cfg.imputed_max_prefill_size, itemsize=itemsize, free_bytes=free_bytes,
+                             reserve_bytes=int(cfg.cache_memory_reserve_gib * (1 << 30)))
+    return CacheManager(requirements, n_pages=counts, page_size=cfg.page_size, max_seqs=cfg.max_seqs,
+                        max_pages_per_seq=cfg.max_pages_per_seq)

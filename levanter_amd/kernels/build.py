@@ -54,7 +54,7 @@ def lib_name(unit: str) -> str:
     return f"liblevanter_amd_{unit}.so"
 
 
-# -packed-fp32-ops off: packed 32-bit float instructions are not to be generated on this hardware pool
+# -packed-fp32-ops off: no packed 32-bit float instructions (v_pk_*_f32) are generated; some forms have given wrong results on MI355X
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}",
     "-O3",

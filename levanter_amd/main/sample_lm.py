@@ -98,7 +98,7 @@ def main(config: SampleLmConfig) -> int:
     else:
         with open(config.random_config) as f:
             engine = InferenceEngine.from_config(LmConfig.from_dict(json.load(f)), config.random_seed, ecfg)
-    print(f"Model ready in {time.time() - t0:.2f} seconds.")
+    print(f"model loaded in {time.time() - t0:.2f} s ({ecfg.compute_dtype})", flush=True)
 
     tokenizer = _load_tokenizer(config.tokenizer, config.hf_checkpoint)
     if config.prompt_ids is not None:
@@ -122,8 +122,9 @@ def main(config: SampleLmConfig) -> int:
 
     base_key = make_key(ecfg.seed)
     for r in range(config.n_rounds):
-        for i, toks in enumerate(prompt_ids):
-            print(f"Prompt {i}: {toks}")
+        if r == 0:
+            for i, toks in enumerate(prompt_ids):
+                print(f"prompt {i} ({len(toks)} tokens): {toks}")
         time_in = time.time()
         reqs = [Request(prompt_tokens=toks, request_id=ridx,
                         decode_params=SeqDecodingParams(max_num_tokens=len(toks) + config.max_new_tokens, stop_tokens=stop,
@@ -131,12 +132,13 @@ def main(config: SampleLmConfig) -> int:
                         n_generations=config.n_generations)
                 for ridx, toks in enumerate(prompt_ids)]
         result = engine.generate(reqs)
-        print(f"Round {r} took {time.time() - time_in:.2f} seconds, generated {result.total_generated} tokens in "
-              f"{len(result.tokens)} sequences.")
+        dt = time.time() - time_in
+        print(f"round {r}: {result.total_generated} tokens in {len(result.tokens)} sequences, {dt:.2f} s "
+              f"({result.total_generated / max(dt, 1e-9):.1f} tok/s)", flush=True)
         for seq_id, out in enumerate(result.tokens):
-            print(f"Tokens for sequence {seq_id} (len: {len(out)}: {out}")
+            print(f"round {r} sequence {seq_id} ({len(out)} tokens, {result.finish_reasons[seq_id]}): {out}")
             if tokenizer is not None:
-                print(f"Generated text for {seq_id}: {tokenizer.decode(out, skip_special_tokens=True)}")
+                print(f"round {r} sequence {seq_id} text: {tokenizer.decode(out, skip_special_tokens=True)}")
     return 0
 
 

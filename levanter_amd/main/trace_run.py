@@ -33,6 +33,8 @@ def main(argv=None) -> int:
     config, model = load_model(args.model, env)
     ps = args.page_size
     n_pages = max(1, (args.max_tokens + ps - 1) // ps)
+    if 64 % ps != 0 and ps % 64 != 0:  # counts are rounded to 64, pages are not: every live request may need one page more
+        n_pages += args.max_seqs
     longest = args.max_tokens if model.max_positions is None else min(args.max_tokens, model.max_positions)
     ecfg = InferenceEngineConfig(max_pages=n_pages, max_seqs=args.max_seqs, page_size=ps,
                                  max_pages_per_seq=max(1, (longest + ps - 1) // ps), compute_dtype=args.dtype)

@@ -82,7 +82,9 @@ def gpt2_model_spec(cfg: Gpt2Config) -> ModelSpec:
         head=head,
         max_positions=cfg.n_positions,
         strip_prefixes=("transformer.",),
-        # the causal-mask buffers of GPT-2 checkpoints and a stored copy of the tied head
-        ignored_tensors=(r"h\.\d+\.attn\.bias", r"h\.\d+\.attn\.masked_bias", r"lm_head\.weight"),
+        # the causal-mask buffers of GPT-2 checkpoints
+        ignored_tensors=(r"h\.\d+\.attn\.bias", r"h\.\d+\.attn\.masked_bias"),
+        # the head is the token table (gpt2.py:361-362): a stored head must be that table
+        stored_copies={"lm_head.weight": "wte.weight"},
         init_std=cfg.initializer_range,
     )

@@ -66,7 +66,10 @@ class ModelSpec:
     strip_prefixes: Tuple[str, ...] = ()
     """Checkpoint name prefixes that may stand before every tensor name and are dropped."""
     ignored_tensors: Tuple[str, ...] = ()
-    """Regular expressions of checkpoint tensors that are not parameters (masks, a stored copy of a tied head)."""
+    """Regular expressions of checkpoint tensors that are not parameters (masks and other buffers)."""
+    stored_copies: Dict[str, str] = field(default_factory=dict)
+    """Checkpoint tensors that may be present as a second copy of a parameter (a stored tied head): name -> the tensor
+    it must equal. A copy that differs is an error: the model would not compute what the file's author computed."""
     init_std: float = 0.02
 
     def all_tensors(self) -> Dict[str, TensorSpec]:

@@ -25,8 +25,10 @@ from .safetensors_io import SafetensorsError, open_model_files
 class WeightsError(ValueError):
     """A checkpoint that does not fit the model: lists missing, unexpected and misshapen tensors."""
 
-    def __init__(self, model_dir: str, missing: List[str], unexpected: List[str], wrong_shape: List[str], wrong_kind: List[str]):
+    def __init__(self, model_dir: str, missing: List[str], unexpected: List[str], wrong_shape: List[str], wrong_kind: List[str],
+                 differing_copies: List[str] = ()):
         self.missing, self.unexpected, self.wrong_shape, self.wrong_kind = missing, unexpected, wrong_shape, wrong_kind
+        self.differing_copies = list(differing_copies)
         lines = [f"checkpoint in {model_dir!r} does not fit the model:"]
         if missing:
             lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
@@ -36,6 +38,8 @@ class WeightsError(ValueError):
             lines.append(f"  wrong shapes ({len(wrong_shape)}): " + "; ".join(wrong_shape))
         if wrong_kind:
             lines.append(f"  wrong dtypes ({len(wrong_kind)}): " + "; ".join(wrong_kind))
+        if differing_copies:
+            lines.append(f"  stored copies that differ from their tensor ({len(differing_copies)}): " + "; ".join(differing_copies))
         super().__init__("\n".join(lines))
 
 
@@ -57,7 +61,8 @@ def load_tensors(model_dir: str, spec: ModelSpec, device: str | torch.device = "
         expected = spec.all_tensors()
         ignored = [re.compile(p) for p in spec.ignored_tensors]
         missing = [n for n in expected if n not in where]
-        unexpected = [n for n in where if n not in expected and not any(r.fullmatch(n) for r in ignored)]
+        copies = {n: of for n, of in spec.stored_copies.items() if n in where}
+        unexpected = [n for n in where if n not in expected and n not in copies and not any(r.fullmatch(n) for r in ignored)]
         wrong_shape, wrong_kind = [], []
         for n, ts in expected.items():
             if n not in where:
@@ -69,8 +74,17 @@ def load_tensors(model_dir: str, spec: ModelSpec, device: str | torch.device = "
             is_float = dtype.is_floating_point
             if (ts.kind == "float") != is_float:
                 wrong_kind.append(f"{n}: file has {dtype}, the model needs a{'n integer' if ts.kind == 'int' else ' real'} tensor")
-        if missing or unexpected or wrong_shape or wrong_kind:
-            raise WeightsError(model_dir, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind)
+        differing = []
+        for n, of in copies.items():  # e.g. the stored head of a model whose head is its token table
+            if of not in where:
+                continue
+            (f, key), (f0, key0) = where[n], where[of]
+            if f.info(key)[1] != f0.info(key0)[1]:
+                differing.append(f"{n}: file has {list(f.info(key)[1])}, {of} has {list(f0.info(key0)[1])}")
+            elif not torch.equal(f.tensor(key).float(), f0.tensor(key0).float()):
+                differing.append(f"{n} is not equal to {of} (the model uses {of} for both)")
+        if missing or unexpected or wrong_shape or wrong_kind or differing:
+            raise WeightsError(model_dir, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind, differing)
         out: Dict[str, torch.Tensor] = {}
         for n, ts in expected.items():
             f, key = where[n]

@@ -151,3 +151,103 @@ def test_random_orders_of_requests_keep_the_books(seed):
     c.reset()
     c.check_invariants()
     assert all(g.pool.n_free == g.pool.n_pages for g in c.groups) and c.n_free_slots == 4
+
+
+# ---- how many pages each group gets -------------------------------------------------------------------------------
+def test_pages_per_group_fixed_none_and_windowed():
+    from levanter_amd.cache import pages_per_group
+
+    full, win = (PagedKv(2, 32), 3), (PagedKv(2, 32, window=40), 2)
+    kw = dict(page_size=16, max_seqs=4, max_pages_per_seq=64, longest_portion=100, itemsize=2)
+    assert pages_per_group([full], max_pages=None, **kw) == [4 * 64]
+    assert pages_per_group([full], max_pages=50, **kw) == [50]
+    # a window of 40 keys and portions of up to 100 tokens touch ceil(140 / 16) + 1 = 10 pages a request
+    assert pages_per_group([full, win], max_pages=None, **kw) == [256, 40]
+    assert pages_per_group([full, win], max_pages=30, **kw) == [30, 30]  # never more than was asked for
+    assert pages_per_group([(PagedKv(2, 32, window=5000), 1)], max_pages=None, **kw) == [256]  # nor than the tables hold
+
+
+def test_pages_per_group_auto_takes_what_the_weights_left():
+    from levanter_amd.cache import pages_per_group
+    from levanter_amd.cache.sizing import GIB, group_page_bytes
+
+    full, win = (PagedKv(8, 128), 32), (PagedKv(8, 128, window=1024), 4)
+    kw = dict(page_size=16, max_seqs=64, max_pages_per_seq=512, longest_portion=2048, itemsize=2)
+    pb_full, pb_win = group_page_bytes(*full, 16, 2), group_page_bytes(*win, 16, 2)
+    assert pb_full == 2 * 32 * 8 * 128 * 16 * 2
+    free = 40 * GIB
+    got = pages_per_group([full, win], max_pages="auto", free_bytes=lambda: free, reserve_bytes=8 * GIB, **kw)
+    n_win = 64 * ((1024 + 2048 + 15) // 16 + 1)
+    assert got[1] == n_win
+    assert got[0] == (free - 8 * GIB - n_win * pb_win) // pb_full
+    assert got[0] * pb_full + got[1] * pb_win <= free - 8 * GIB < (got[0] + 1) * pb_full + got[1] * pb_win
+    # plenty of memory: no more than every request at full length
+    assert pages_per_group([full], max_pages="auto", free_bytes=lambda: 10_000 * GIB, **kw) == [64 * 512]
+    # too little for one request of full length beside the reserve: an error that says how much is needed
+    with pytest.raises(MemoryError, match="GiB are free"):
+        pages_per_group([full], max_pages="auto", free_bytes=lambda: 8 * GIB + GIB // 2, reserve_bytes=8 * GIB, **kw)
+    with pytest.raises(ValueError, match="query"):
+        pages_per_group([full], max_pages="auto", **kw)
+
+
+def test_engine_cache_sized_from_a_stubbed_memory_query():
+    from levanter_amd.config import InferenceEngineConfig, LmConfig
+    from levanter_amd.engine.loading import make_cache
+    from levanter_amd.cache.sizing import GIB
+    from tiny_configs import TINY_B
+
+    class Model:  # what make_cache asks of a model
+        def cache_requirements(self):
+            spec = LmConfig.from_dict(TINY_B).model_spec()
+            return [(e.cache, PagedKv(3, 32)) for e in spec.plan]
+
+    cfg = InferenceEngineConfig(max_pages="auto", max_seqs=64, max_pages_per_seq=4096, page_size=16, compute_dtype="float32",
+                                cache_memory_reserve_gib=1.0)
+    cache = make_cache(Model(), cfg, free_bytes=lambda: 3 * GIB)
+    page_bytes = 2 * 3 * 3 * 32 * 16 * 4  # keys and values, 3 layers, 3 heads of 32, 16 tokens, float32
+    assert [g.pool.n_pages for g in cache.groups] == [2 * GIB // page_bytes]
+    with pytest.raises(Exception, match="auto"):
+        InferenceEngineConfig(max_pages="most")
+
+
+def test_padding_tokens_of_a_replayed_step_beside_a_window_that_has_moved_on():
+    """Steps of single tokens are filled up to a multiple of 8 with padding tokens (request row 0, position 0, written
+    nowhere). In a group with a window the first request's block 0 has long been given back: the padding names a
+    block without a page, which the attention kernels mask. Every key that a real token can see has a page."""
+    import torch
+
+    from levanter_amd.engine.step import ModelRunner, StepEntry, graph_batch_bucket
+    from levanter_amd.parts import BuildEnv
+    from levanter_amd.parts.spec import PlanEntry
+
+    class Model:
+        vocab_size, max_positions, plan = 50, None, [PlanEntry(0, 0), PlanEntry(1, 1)]
+
+        def cache_requirements(self):
+            return [(0, PagedKv(1, 16)), (1, PagedKv(1, 16, window=20))]
+
+    window = 20
+    cache = CacheManager(Model().cache_requirements(), n_pages=[40, 16], page_size=16, max_seqs=8, max_pages_per_seq=8)
+    runner = ModelRunner(Model(), cache, BuildEnv(torch.float32, torch.device("cpu"), None), allocate=False)
+    handles = [cache.open(i) for i in range(5)]
+    for h in handles:
+        cache.extend(h, 60)
+        cache.advance(h, 60)
+    assert cache.groups[1].block_tables[handles[0].slot, 0] == NO_PAGE  # behind the window
+    entries = [StepEntry(h, [7], [0]) for h in handles]
+    for h in handles:
+        cache.extend(h, 1)
+    b = runner._build_host(entries, pad_blocks=1, pad_batch=True)
+    assert b.n_tokens == graph_batch_bucket(5) == 8 and b.n_rows_real == 5
+    view = lambda i: b.host[b.offs[i]:b.offs[i] + b.sizes[i]]
+    positions, token_seq = view(1), view(2)
+    assert list(positions[5:]) == [0, 0, 0] and list(token_seq[5:]) == [0, 0, 0]
+    for gi, g in enumerate(cache.groups):
+        bt = view(7 + 2 * gi).reshape(b.n_seqs, b.max_blocks)
+        dest = view(8 + 2 * gi)
+        assert (dest[:5] >= 0).all() and (dest[5:] == -1).all()
+        w = g.requirement.window
+        for t in range(5):  # real tokens: every visible key has a page
+            lo = 0 if w is None else max(0, positions[t] - w + 1)
+            assert (bt[token_seq[t], lo // 16: positions[t] // 16 + 1] != NO_PAGE).all()
+    assert view(7 + 2 * 1).reshape(b.n_seqs, b.max_blocks)[0, 0] == NO_PAGE  # what the padding tokens point at

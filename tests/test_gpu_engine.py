@@ -315,6 +315,20 @@ def _run_cut(spec, tensors, dtype, toks, cuts, n_pages=16, state_checks=None):
     return torch.cat(out), cache, h
 
 
+def _plain_logits_with_a_window_in_layer_1(w, toks, W, rounding=lambda x: x):
+    """Tiny A with a window of W keys in its second layer: layer 0 sees everything."""
+    n = len(toks)
+    x = P.plain_embed(torch.tensor(toks), torch.arange(n), w["wte.weight"], w["wpe.weight"])
+    for i in range(2):
+        p = f"h.{i}."
+        hh = rounding(P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5))
+        q, k, v = P.plain_split_qkv(rounding(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"])), 4)
+        o = rounding(P.plain_causal_attention(q, k, v, window=W if i == 1 else None, rounding=rounding))
+        x = x + P.plain_linear(o.transpose(0, 1).reshape(n, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+        x = x + P.plain_mlp(rounding(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5)), w, p, TINY_A, rounding)
+    return rounding(P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5)) @ w["wte.weight"].T
+
+
 def test_window_layer_has_its_own_pages_and_gives_them_back():
     d = write_model(TINY_A, 0, torch.float32)
     w = read_weights(d)
@@ -322,22 +336,61 @@ def test_window_layer_has_its_own_pages_and_gives_them_back():
     W = 20
     spec = _toy_spec(window=W)
     toks = torch.randint(0, 512, (100,), generator=torch.Generator().manual_seed(3)).tolist()
-    # plain: layer 0 sees everything, layer 1 a window of 20 keys
-    x = P.plain_embed(torch.tensor(toks), torch.arange(100), w["wte.weight"], w["wpe.weight"])
-    for i in range(2):
-        p = f"h.{i}."
-        hh = P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5)
-        q, k, v = P.plain_split_qkv(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"]), 4)
-        o = P.plain_causal_attention(q, k, v, window=W if i == 1 else None)
-        x = x + P.plain_linear(o.transpose(0, 1).reshape(100, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
-        x = x + P.plain_mlp(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5), w, p, TINY_A)
-    want = P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+    want = _plain_logits_with_a_window_in_layer_1(w, toks, W)
     for cuts in ([100], [37, 2, 30, 1, 1, 1, 28], [1] * 100):
         got, cache, h = _run_cut(spec, t32, "float32", toks, cuts, n_pages=7)
         torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-5)
         assert len(cache.groups) == 2
         g_all, g_win = cache.groups if cache.groups[0].requirement.window is None else cache.groups[::-1]
         assert len(g_all.pages_held(h.slot)) == 7 and len(g_win.pages_held(h.slot)) <= 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_layer_beside_other_requests_in_replayed_steps(dtype):
+    """Six requests decode together past their windows: steps of single tokens are filled up to eight with padding
+    tokens and replayed as a graph; the padding names the first request's block 0, which its window has given back
+    long ago. The window group's pool is so small that pages go round. Every row against the plain implementation."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import make_cache
+    from levanter_amd.parts import DecoderLm
+
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    d = write_model(TINY_A, 0, store)
+    w = read_weights(d)
+    W = 20
+    env = _env(dtype)
+    model = DecoderLm(_toy_spec(window=W), {k: v.to(store) for k, v in w.items()}, env)
+    cfg = InferenceEngineConfig(max_pages=48, max_seqs=8, page_size=16, max_pages_per_seq=8, compute_dtype=dtype, max_prefill_size=40)
+    cache = make_cache(model, cfg)
+    g_all, g_win = cache.groups if cache.groups[0].requirement.window is None else cache.groups[::-1]
+    assert g_all.pool.n_pages == 48 and g_win.pool.n_pages == 8 * ((W + 40 + 15) // 16 + 1)  # sized by what a window can hold
+    runner = ModelRunner(model, cache, env)
+    assert runner.use_graphs
+    gen = torch.Generator().manual_seed(9)
+    lens = [100, 90, 75, 110, 64, 101]
+    seqs = [torch.randint(0, 512, (n,), generator=gen).tolist() for n in lens]
+    rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    want = [_plain_logits_with_a_window_in_layer_1(w, t, W, rounding) for t in seqs]
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == "float32" else dict(rtol=2e-2, atol=8e-3)
+    handles = [cache.open(i) for i in range(6)]
+    done = [0] * 6
+    for i, h in enumerate(handles):  # prompts of 30 .. 40 tokens, two at a time
+        n = 30 + 2 * i
+        got = runner.step([StepEntry(h, seqs[i][:n], list(range(n)))]).cpu()
+        torch.testing.assert_close(got.double(), want[i][:n], **tol)
+        done[i] = n
+    worst_held = 0
+    while any(done[i] < lens[i] for i in range(6)):
+        live = [i for i in range(6) if done[i] < lens[i]]
+        got = runner.step([StepEntry(handles[i], [seqs[i][done[i]]], [0]) for i in live]).cpu()
+        for r, i in enumerate(live):
+            torch.testing.assert_close(got[r].double(), want[i][done[i]], **tol, msg=lambda m: f"request {i} position {done[i]}: {m}")
+            done[i] += 1
+        cache.check_invariants()
+        worst_held = max(worst_held, max(len(g_win.pages_held(h.slot)) for h in handles))
+    assert worst_held <= 3 and g_win.block_tables[handles[0].slot, 0] == -1
+    assert any(not isinstance(v, str) for v in runner._graphs.values())  # steps were replayed from a recorded graph
 
 
 def test_a_layer_named_twice_and_a_layer_reading_anothers_cache():

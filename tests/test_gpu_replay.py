@@ -28,10 +28,10 @@ TOL_F32 = dict(rtol=1e-4, atol=1e-5)
 TOL_BF16 = dict(rtol=2e-2, atol=8e-3)
 
 
-def run_trace(model_dir, dtype, steps, max_tokens):
+def run_trace(model_dir, dtype, steps, max_tokens, extra=()):
     out = tempfile.mkdtemp(prefix="lev_trace_")
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype, "--out", out,
-           "--max-tokens", str(max_tokens)]
+           "--max-tokens", str(max_tokens), *extra]
     p = subprocess.run(cmd, input=TR.to_jsonl(steps), capture_output=True, text=True, timeout=600)
     assert p.returncode == 0, p.stderr[-3000:]
     assert p.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
@@ -42,21 +42,29 @@ def read_step(out, step, vocab):
     return torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
 
 
+LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [130, 66, 35, 97, 64, 18]}
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_all_cuttings(name, dtype):
     raw, seed = TINY[name]
+    check_all_cuttings(f"trace_run {name}", raw, seed, dtype, LENGTHS[name])
+
+
+def check_all_cuttings(label, raw, seed, dtype, lengths, page_size=16):
+    """The requests whole, with the last 32 tokens one by one, in portions of changing size and twice mixed in a pool
+    of exactly the peak need, through ``bin/trace_run``; every wanted row against the plain implementation."""
     store = torch.float32 if dtype == "float32" else torch.bfloat16
     d = write_model(raw, seed, store)
     weights = read_weights(d)
-    lengths = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [130, 66, 35, 97, 64, 18]}[name]
     reqs = TR.random_requests(raw["vocab_size"], lengths, seed + 10)
     rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
     plain = {rid: P.plain_logits(weights, raw, torch.tensor(t), rounding=rounding) for rid, t in reqs.items()}
     steps = TR.number(TR.trace_whole(reqs) + TR.trace_prefill_then_singles(reqs) + TR.trace_portions(reqs)
                       + TR.trace_mixed(reqs, seed=3) + TR.trace_mixed(reqs, seed=4, prefix="n"))
-    max_tokens = TR.peak_tokens(steps)
-    out = run_trace(d, dtype, steps, max_tokens)
+    max_tokens = TR.peak_tokens(steps, round_to=64 if 64 % page_size == 0 else page_size)  # whole pages of every request
+    out = run_trace(d, dtype, steps, max_tokens, extra=() if page_size == 16 else ("--page-size", str(page_size)))
     want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
     tol = TOL_F32 if dtype == "float32" else TOL_BF16
     worst = 0.0
@@ -67,7 +75,7 @@ def test_trace_run_all_cuttings(name, dtype):
             got = read_step(out, k, raw["vocab_size"])
             worst = max(worst, float((got.double() - want[k]).abs().max()))
             torch.testing.assert_close(got.double(), want[k], **tol, msg=lambda m: f"step {k} {s['entries'][0]['id']}: {m}")
-    print(f"trace_run {name} {dtype}: worst abs difference {worst:.3e}")
+    print(f"{label} {dtype}: worst abs difference {worst:.3e}")
     if dtype == "bfloat16":
         # and against the 32-bit plain implementation: the greedy token agrees wherever its margin is clear
         plain32 = {rid: P.plain_logits(weights, raw, torch.tensor(t)) for rid, t in reqs.items()}

@@ -34,7 +34,9 @@ def test_activations_are_the_library_ones_and_not_each_other():
     torch.testing.assert_close(P.plain_activation("silu")(u), F.silu(u))
     torch.testing.assert_close(P.plain_activation("swish")(u), F.silu(u))
     torch.testing.assert_close(P.plain_activation("relu")(u), F.relu(u))
-    torch.testing.assert_close(P.plain_activation("quick_gelu")(u), u * torch.sigmoid(1.702 * u))
+    # u sigmoid(a u) = silu(a u) / a: quick_gelu through the library's silu
+    torch.testing.assert_close(P.plain_activation("quick_gelu")(u), F.silu(1.702 * u) / 1.702, rtol=1e-12, atol=1e-12)
+    assert float((P.plain_activation("quick_gelu")(u) - F.gelu(u)).abs().max()) > 1e-3  # and it is not a gelu
     # the two gelus differ where |u| is about 2: a swapped option cannot pass both checks above
     diff = (P.plain_activation("gelu")(u) - P.plain_activation("gelu_new")(u)).abs().max()
     assert 1e-4 < float(diff) < 1e-2
@@ -55,15 +57,42 @@ def test_linear_layout_is_in_out():
     assert P.plain_linear(x, w2, None).shape == (3, 20)
 
 
-def test_qkv_split_order_and_head_columns():
-    n_head, hd, t = 3, 32, 5
+def test_qkv_roles_and_head_columns_through_library_attention():
+    """Which third of the fused projection is the query, the key and the value, and which columns are a head. The
+    order (q, k, v), then heads, then head size is the reference's (src/levanter/models/gpt2.py:172-174,184-185 with
+    the flattening of src/levanter/compat/hf_checkpoints.py); no stored numbers of the reference cover it, so against
+    another implementation this order is "parity unpinned". What is pinned: each third plays its role. With the first
+    third's weight zero and its bias a constant vector c, every query is c: scores depend on the key only, and the
+    result is the library's attention with q = c. Were the first third the keys, scores would not depend on the key
+    and every row would be a running mean of the values; were it the values, the output would be c."""
+    n_head, hd, t = 3, 32, 7
     d = n_head * hd
+    g = torch.Generator().manual_seed(11)
+    h = torch.randn(t, d, dtype=D64, generator=g)
+    w = torch.randn(d, 3 * d, dtype=D64, generator=g) * 0.3
+    b = torch.randn(3 * d, dtype=D64, generator=g)
+    c = torch.randn(d, dtype=D64, generator=g) * 2
+    w[:, :d] = 0
+    b[:d] = c
+    q, k, v = P.plain_split_qkv(P.plain_linear(h, w, b), n_head)
+    got = P.plain_causal_attention(q, k, v)
+    heads = lambda m: m.reshape(t, n_head, hd).transpose(0, 1)  # columns of a third: head-major
+    want = F.scaled_dot_product_attention(heads(c.expand(t, d)), heads(h @ w[:, d:2 * d] + b[d:2 * d]),
+                                          heads(h @ w[:, 2 * d:] + b[2 * d:]), is_causal=True)
+    torch.testing.assert_close(got, want, rtol=1e-10, atol=1e-10)
+    running_mean = torch.cumsum(heads(h @ w[:, 2 * d:] + b[2 * d:]), 1) / torch.arange(1, t + 1, dtype=D64).view(1, t, 1)
+    assert not torch.allclose(got, running_mean, atol=1e-3)
+    # the last third is the value: with it zero (weight and bias) the output vanishes whatever q and k are
+    w2, b2 = w.clone(), b.clone()
+    w2[:, 2 * d:] = 0
+    b2[2 * d:] = 0
+    q, k, v = P.plain_split_qkv(P.plain_linear(h, w2, b2), n_head)
+    assert float(P.plain_causal_attention(q, k, v).abs().max()) == 0.0
+    # head-major columns inside a third: the split of a counted matrix
     qkv = torch.arange(t * 3 * d, dtype=D64).reshape(t, 3 * d)
     q, k, v = P.plain_split_qkv(qkv, n_head)
     assert q.shape == (n_head, t, hd)
-    torch.testing.assert_close(q[1, 2], qkv[2, 0 * d + 1 * hd: 0 * d + 2 * hd])
     torch.testing.assert_close(k[2, 4], qkv[4, 1 * d + 2 * hd: 1 * d + 3 * hd])
-    torch.testing.assert_close(v[0, 3], qkv[3, 2 * d: 2 * d + hd])
 
 
 def test_attention_is_library_sdpa():
@@ -130,9 +159,19 @@ def test_whole_model_shapes_causality_and_tied_head(config, seed):
     logits2 = P.plain_logits(w, config, toks2)
     torch.testing.assert_close(logits2[:12], logits[:12], rtol=1e-12, atol=1e-12)
     assert not torch.allclose(logits2[12:], logits[12:])
-    # the head is the token table: scaling wte rows scales embedding and head alike
-    hidden = P.plain_hidden(w, config, toks)
-    torch.testing.assert_close(logits, hidden @ w["wte.weight"].T)
+    # the head is the token table (src/levanter/models/gpt2.py:361-362): changing the row of a token that is not in the
+    # prompt changes nothing before the head, so exactly that token's logits move, by hidden . delta
+    absent = next(v for v in range(s["V"]) if v not in set(toks.tolist()))
+    w3 = dict(w)
+    delta = torch.linspace(-1, 1, s["D"], dtype=w["wte.weight"].dtype)
+    w3["wte.weight"] = w["wte.weight"].clone()
+    w3["wte.weight"][absent] += delta
+    logits3 = P.plain_logits(w3, config, toks)
+    moved = (logits3 - logits).abs().max(0).values
+    assert float(moved[absent]) > 1e-3
+    moved[absent] = 0
+    assert float(moved.max()) == 0.0
+    torch.testing.assert_close(logits3[:, absent] - logits[:, absent], P.plain_hidden(w, config, toks) @ delta, rtol=1e-9, atol=1e-9)
 
 
 def test_pre_norm_placement_and_layer_scale():

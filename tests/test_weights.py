@@ -45,6 +45,27 @@ def test_float32_stays_float32_and_prefix_is_dropped(tmp_path):
     assert all(torch.equal(t2[k], t[k]) for k in t)
 
 
+def test_a_stored_head_must_be_the_token_table(tmp_path):
+    """GPT-2's head is its token table (src/levanter/models/gpt2.py:361-362). A checkpoint may carry ``lm_head.weight``
+    as a copy; one that differs (an untied fine-tune) would give other logits than its author's and is refused."""
+    d = write_model(TINY_A, 0, torch.float32)
+    spec = LmConfig.load(d).model_spec()
+    t = load_tensors(d, spec)
+    LmConfig.load(d).save(str(tmp_path))
+    save_file({**t, "lm_head.weight": t["wte.weight"].clone()}, str(tmp_path / "model.safetensors"))
+    t2 = load_tensors(str(tmp_path), spec)
+    assert sorted(t2) == sorted(t) and torch.equal(t2["wte.weight"], t["wte.weight"])
+    other = t["wte.weight"].clone()
+    other[3, 5] += 1e-3
+    save_file({**t, "lm_head.weight": other}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError, match="lm_head.weight is not equal to wte.weight") as e:
+        load_tensors(str(tmp_path), spec)
+    assert e.value.differing_copies and not e.value.unexpected
+    save_file({**t, "lm_head.weight": other[:-1]}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightsError, match=r"lm_head.weight: file has \[511, 64\]"):
+        load_tensors(str(tmp_path), spec)
+
+
 def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
     d = write_model(TINY_A, 0, torch.float32)
     spec = LmConfig.load(d).model_spec()

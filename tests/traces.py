@@ -17,22 +17,31 @@ def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, 
     return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
 
 
-def _entry(rid, toks, start, n, want_all=True):
-    return {"id": rid, "tokens": toks[start:start + n], "want": list(range(n)) if want_all else []}
+def want_all(n):
+    return list(range(n))
 
 
-def trace_whole(reqs, prefix="w"):
+def want_ends(n):
+    """The first, the middle and the last two places of a portion: for models whose vocabulary makes every row costly."""
+    return sorted({0, n // 2, max(0, n - 2), n - 1})
+
+
+def _entry(rid, toks, start, n, want=want_all):
+    return {"id": rid, "tokens": toks[start:start + n], "want": want(n)}
+
+
+def trace_whole(reqs, prefix="w", want=want_all):
     """Each request alone, all its tokens in one step."""
-    return [{"entries": [_entry(prefix + rid, toks, 0, len(toks))], "end": [prefix + rid]} for rid, toks in reqs.items()]
+    return [{"entries": [_entry(prefix + rid, toks, 0, len(toks), want)], "end": [prefix + rid]} for rid, toks in reqs.items()]
 
 
-def trace_prefill_then_singles(reqs, n_single=32, prefix="s"):
+def trace_prefill_then_singles(reqs, n_single=32, prefix="s", want=want_all):
     """All but the last ``n_single`` tokens in one step, then one token a step."""
     steps = []
     for rid, toks in reqs.items():
         n = len(toks)
         k = max(1, n - n_single)
-        steps.append({"entries": [_entry(prefix + rid, toks, 0, k)], "end": []})
+        steps.append({"entries": [_entry(prefix + rid, toks, 0, k, want)], "end": []})
         for i in range(k, n):
             steps.append({"entries": [_entry(prefix + rid, toks, i, 1)], "end": [prefix + rid] if i == n - 1 else []})
         if k == n:
@@ -40,21 +49,21 @@ def trace_prefill_then_singles(reqs, n_single=32, prefix="s"):
     return steps
 
 
-def trace_portions(reqs, prefix="p"):
+def trace_portions(reqs, prefix="p", sizes=PORTION_SIZES, want=want_all):
     """Portions of changing size, down to two tokens."""
     steps = []
     j = 0
     for rid, toks in reqs.items():
         i, n = 0, len(toks)
         while i < n:
-            size = min(PORTION_SIZES[j % len(PORTION_SIZES)], n - i)
+            size = min(sizes[j % len(sizes)], n - i)
             j += 1
-            steps.append({"entries": [_entry(prefix + rid, toks, i, size)], "end": [prefix + rid] if i + size == n else []})
+            steps.append({"entries": [_entry(prefix + rid, toks, i, size, want)], "end": [prefix + rid] if i + size == n else []})
             i += size
     return steps
 
 
-def trace_mixed(reqs, seed=0, max_live=4, prefix="m", decode_tail=12):
+def trace_mixed(reqs, seed=0, max_live=4, prefix="m", decode_tail=12, sizes=(2, 3, 5, 7, 16, 17, 30), want=want_all):
     """Up to ``max_live`` live requests; portions of some beside single tokens of others in one step;
     requests are sometimes left out of a step; a finished request's place is taken by the next."""
     rng = random.Random(seed)
@@ -74,8 +83,8 @@ def trace_mixed(reqs, seed=0, max_live=4, prefix="m", decode_tail=12):
             if i >= n - decode_tail:
                 size = 1
             else:
-                size = min(rng.choice([2, 3, 5, 7, 16, 17, 30]), n - decode_tail - i)
-            entries.append(_entry(rid, toks, i, size))
+                size = min(rng.choice(list(sizes)), n - decode_tail - i)
+            entries.append(_entry(rid, toks, i, size, want))
             if i + size == n:
                 end.append(rid)
                 del live[rid]
