@@ -185,19 +185,21 @@ class ModelRunner:
         if pad_blocks > 1:
             max_blocks = min((max_blocks + pad_blocks - 1) // pad_blocks * pad_blocks, cache.max_pages_per_seq)
         n_groups = len(cache.groups)
-        sizes = [T, T, T, S, len(rows), len(tiles), len(decode)] + [S * max_blocks, T] * n_groups
+        token_slots = seq_slots[token_seq].astype(np.int32)
+        token_slots[n_real_tokens:] = -1  # ghosts belong to nobody: a mixer with state of its own leaves them out
+        sizes = [T, T, T, S, len(rows), len(tiles), len(decode), T] + [S * max_blocks, T] * n_groups
         offs = np.concatenate([[0], np.cumsum([(x + 3) // 4 * 4 for x in sizes])]).astype(np.int64)
         host = np.zeros(int(offs[-1]), np.int32)
-        for i, arr in enumerate((tokens, positions, token_seq, seq_slots, rows, tiles, decode)):
+        for i, arr in enumerate((tokens, positions, token_seq, seq_slots, rows, tiles, decode, token_slots)):
             host[offs[i]:offs[i] + sizes[i]] = arr
         for gi, g in enumerate(cache.groups):
             bt = g.block_tables[seq_slots, :max_blocks]
-            host[offs[7 + 2 * gi]:offs[7 + 2 * gi] + S * max_blocks] = bt.reshape(-1)
+            host[offs[N_FIXED + 2 * gi]:offs[N_FIXED + 2 * gi] + S * max_blocks] = bt.reshape(-1)
             pages = g.block_tables[seq_slots[token_seq], positions // ps]
             assert (pages[:n_real_tokens] != NO_PAGE).all(), "a new token has no page"
             dest = pages * ps + positions % ps
             dest[n_real_tokens:] = -1  # ghosts are written nowhere
-            host[offs[8 + 2 * gi]:offs[8 + 2 * gi] + T] = dest
+            host[offs[N_FIXED + 1 + 2 * gi]:offs[N_FIXED + 1 + 2 * gi] + T] = dest
         return HostBatch(host=host, sizes=sizes, offs=[int(o) for o in offs], n_tokens=T, n_seqs=S, n_rows=len(rows),
                          n_tiles=len(tiles) // 2, n_decode=len(decode), max_blocks=max_blocks, max_kv=max_blocks * ps,
                          run_lengths=run_lengths, first_positions=first_positions, slots=[int(x) for x in seq_slots[:len(entries)]],
@@ -214,10 +216,10 @@ class ModelRunner:
             decode_tokens=view(6) if b.n_decode else None, n_decode=b.n_decode,
             max_kv_len=b.max_kv, _workspaces=workspaces)
         ctx = StepContext(kernels=self.env.kernels, dtype=self.env.dtype, device=self.env.device, n_tokens=b.n_tokens,
-                          tokens=view(0), attention=meta, seq_slots=view(3),
+                          tokens=view(0), attention=meta, seq_slots=view(3), token_slots=view(7),
                           host={"run_lengths": b.run_lengths, "first_positions": b.first_positions, "slots": b.slots})
-        group_views = [GroupView(page_size=ps, block_tables=view(7 + 2 * gi).view(b.n_seqs, b.max_blocks), dest=view(8 + 2 * gi))
-                       for gi in range(len(cache.groups))]
+        group_views = [GroupView(page_size=ps, block_tables=view(N_FIXED + 2 * gi).view(b.n_seqs, b.max_blocks),
+                                 dest=view(N_FIXED + 1 + 2 * gi)) for gi in range(len(cache.groups))]
         for unit, g in cache.group_of_unit.items():
             i = g.unit_pos[unit]
             ctx.units[unit] = CacheUnitView(k_pages=None if g.k_pages is None else g.k_pages[i],
@@ -284,6 +286,7 @@ class ModelRunner:
         return entry.logits
 
 
+N_FIXED = 8  # arrays of the step's buffer ahead of the cache groups' (block tables, destinations)
 GRAPH_BLOCK_BUCKET = 16  # block tables of graphed steps are padded to a multiple of this many pages
 MAX_GRAPHS = 48
 

@@ -23,7 +23,7 @@ def gpt2_model_spec(cfg: Gpt2Config) -> ModelSpec:
         tensors = {"weight": TensorSpec(prefix + ".weight", (d,), init="one_plus_normal")}
         if bias:
             tensors["bias"] = TensorSpec(prefix + ".bias", (d,))
-        return PartSpec("layernorm", {"dim": d, "eps": cfg.layer_norm_epsilon, "bias": bias}, tensors)
+        return PartSpec("layernorm", {"dim": d, "eps": cfg.layer_norm_epsilon, "bias": bias}, tensors, family="norm")
 
     def linear_tensors(prefix: str, n_in: int, n_out: int, local: str) -> dict:
         t = {local + ".weight": TensorSpec(prefix + ".weight", (n_in, n_out))}
@@ -52,25 +52,30 @@ def gpt2_model_spec(cfg: Gpt2Config) -> ModelSpec:
                 "rotary": None,
             },
             {**linear_tensors(p + ".attn.c_attn", d, 3 * d, "qkv"), **linear_tensors(p + ".attn.c_proj", d, d, "out")},
+            family="mixer",
         )
         ff = PartSpec(
             "dense_mlp",
             {"dim": d, "inner_dim": f, "activation": cfg.activation_function, "bias": bias, "weight_layout": "in_out"},
             {**linear_tensors(p + ".mlp.c_fc", d, f, "up"), **linear_tensors(p + ".mlp.c_proj", f, d, "down")},
+            family="feed_forward",
         )
-        layers.append(LayerSpec("pre_norm", norm(p + ".ln_1"), mixer, norm(p + ".ln_2"), ff))
+        layers.append(LayerSpec("pre_norm", norm1=norm(p + ".ln_1"), mixer=mixer, norm2=norm(p + ".ln_2"), feed_forward=ff))
 
     position = PartSpec(
         "learned_absolute",
         {"n_positions": cfg.n_positions, "dim": d},
         {"table": TensorSpec("wpe.weight", (cfg.n_positions, d))},
+        family="position",
     )
     embedding = PartSpec(
         "token_embedding",
         {"vocab_size": cfg.vocab_size, "dim": d, "position": position},
         {"table": TensorSpec("wte.weight", (cfg.vocab_size, d))},
+        family="embedding",
     )
-    head = PartSpec("tied_head", {"vocab_size": cfg.vocab_size, "dim": d}, {"table": TensorSpec("wte.weight", (cfg.vocab_size, d))})
+    head = PartSpec("tied_head", {"vocab_size": cfg.vocab_size, "dim": d}, {"table": TensorSpec("wte.weight", (cfg.vocab_size, d))},
+                    family="head")
     return ModelSpec(
         architecture="gpt2",
         vocab_size=cfg.vocab_size,

@@ -16,8 +16,9 @@ import torch
 
 from levanter_amd.cache.requirements import PagedKv
 from .base import BuildEnv, CacheUnitView, Mixer, StepContext
+from .embedding import tensors_of_nested
 from .linear import Linear
-from .registry import MIXERS, POSITION_ENCODINGS
+from .registry import MIXERS, part_class
 from .spec import PartSpec
 
 
@@ -48,7 +49,7 @@ class CausalSelfAttention(Mixer):
         rotary = p.get("rotary")
         self.rotary = None
         if rotary is not None:
-            self.rotary = POSITION_ENCODINGS.get(rotary.kind)(rotary, {k: tensors[k] for k in rotary.tensors}, env)
+            self.rotary = part_class(rotary.kind, rotary.family or "position")(rotary, tensors_of_nested("rotary", tensors), env)
             self.graph_safe = bool(self.rotary.graph_safe)  # the rotation runs inside this mixer's forward
 
     def cache_requirement(self):

@@ -79,6 +79,10 @@ class StepContext:
     attention: AttentionMeta
     seq_slots: torch.Tensor  # int32 [S] state slot of each request in the step
     host: Dict[str, Any]  # "run_lengths", "first_positions", "slots": lists, one entry per request in the step
+    token_slots: Optional[torch.Tensor] = None
+    """int32 [T]: the state slot of each token's request, -1 for the padding tokens of a replayed step (they belong to
+    nobody: a mixer with state of its own must not count them). With ``attention.positions`` and
+    ``attention.token_seq`` this is all a state mixer needs on the device, so that it can be ``graph_safe``."""
     units: Dict[int, CacheUnitView] = field(default_factory=dict)
 
     def empty(self, rows: int, cols: int, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -144,15 +148,52 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
-class Block(Part):
-    """Arranges two norms, a mixer and a feed-forward. ``forward(x, ctx, unit, writes_cache)`` updates ``x`` in place."""
+class Block:
+    """Arranges the parts of a layer around the residual stream. Built from ``parts``: role -> built part, with the
+    roles its description names; ``roles`` lists the ones this block cannot do without. One plan entry has one
+    cache unit: ``cache_requirement()`` says what it holds (by default what the part in the role ``mixer`` asks for).
+    ``forward(x, ctx, unit, writes_cache)`` updates ``x`` in place."""
+
+    kind: str = ""
+    roles: tuple = ()
+
+    def __init__(self, parts: Dict[str, Part]):
+        missing = [r for r in self.roles if r not in parts]
+        if missing:
+            raise ValueError(f"block {self.kind!r} needs the parts {', '.join(self.roles)}; the description lacks {', '.join(missing)}")
+        self.parts = dict(parts)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts.values())
+
+    def cache_requirement(self):
+        mixer = self.parts.get("mixer")
+        return None if mixer is None else mixer.cache_requirement()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """``__call__(ctx) -> x`` float32 ``[T, dim]``: the residual stream's first value, from ``ctx.tokens`` (and
+    positions, if the embedding has a position encoding). ``table``: the token table ``[vocab, dim]`` in the compute
+    dtype, for a head that is tied to it (None if there is no such table). ``max_positions``: the largest sequence
+    length it allows, or None."""
+
+    table: Optional[torch.Tensor] = None
+    max_positions: Optional[int] = None
+
+    def __call__(self, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Head(Part):
-    """``__call__(h [R, dim], ctx) -> logits float32 [R, vocab]``."""
+    """``__call__(h [R, dim], ctx) -> logits float32 [R, vocab]``. ``bind(embedding)`` is called once when the
+    model is built: a tied head takes the embedding's table there; others ignore it."""
+
+    def bind(self, embedding: Embedding) -> None:
+        return None
 
     def __call__(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError

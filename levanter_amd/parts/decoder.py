@@ -13,37 +13,9 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from .base import BuildEnv, StepContext
-from .registry import BLOCKS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS
+from .embedding import nested_tensors
+from .registry import BLOCKS, part_class
 from .spec import ModelSpec, PartSpec
-
-
-def _part_tensors(spec: PartSpec, tensors: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
-    out = {local: tensors[ts.name] for local, ts in spec.tensors.items()}
-    for v in spec.params.values():
-        if isinstance(v, PartSpec):  # a nested part's tensors travel under its own local names
-            out.update(_part_tensors(v, tensors))
-    return out
-
-
-class TokenEmbedding:
-    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
-        self.vocab_size = int(spec.params["vocab_size"])
-        self.dim = int(spec.params["dim"])
-        self.table = tensors[spec.tensors["table"].name].to(env.device, env.dtype).contiguous()
-        pos_spec: Optional[PartSpec] = spec.params.get("position")
-        self.position = None
-        if pos_spec is not None:
-            self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, _part_tensors(pos_spec, tensors), env)
-
-    @property
-    def max_positions(self) -> Optional[int]:
-        return None if self.position is None else self.position.max_positions
-
-    def __call__(self, ctx: StepContext) -> torch.Tensor:
-        x = ctx.empty(ctx.n_tokens, self.dim, torch.float32)
-        pos_table = None if self.position is None else self.position.embedding_table()
-        ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x)
-        return x
 
 
 class DecoderLm:
@@ -52,19 +24,16 @@ class DecoderLm:
         self.env = env
         self.vocab_size = spec.vocab_size
         self.dim = spec.dim
-        self.embedding = TokenEmbedding(spec.embedding, tensors, env)
-        self.blocks = []
-        for layer in spec.layers:
-            norm1 = NORMS.get(layer.norm1.kind)(layer.norm1, _part_tensors(layer.norm1, tensors), env)
-            mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _part_tensors(layer.mixer, tensors), env)
-            norm2 = NORMS.get(layer.norm2.kind)(layer.norm2, _part_tensors(layer.norm2, tensors), env)
-            ff = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward, _part_tensors(layer.feed_forward, tensors), env)
-            self.blocks.append(BLOCKS.get(layer.block)(norm1, mixer, norm2, ff))
+
+        def build(part: PartSpec, family: str = ""):
+            return part_class(part.kind, part.family or family)(part, nested_tensors(part, tensors), env)
+
+        self.embedding = build(spec.embedding, "embedding")
+        self.blocks = [BLOCKS.get(layer.block)({role: build(part) for role, part in layer.parts.items()}) for layer in spec.layers]
         self.plan = list(spec.plan)
-        self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _part_tensors(spec.final_norm, tensors), env)
-        self.head = HEADS.get(spec.head.kind)(spec.head, _part_tensors(spec.head, tensors), env)
-        if hasattr(self.head, "tie"):
-            self.head.tie(self.embedding.table)
+        self.final_norm = build(spec.final_norm, "norm")
+        self.head = build(spec.head, "head")
+        self.head.bind(self.embedding)
         self._check_plan()
 
     def _check_plan(self) -> None:
@@ -80,18 +49,15 @@ class DecoderLm:
             if not e.writes_cache:
                 if e.cache not in owners or owners[e.cache] > i:
                     raise ValueError(f"plan entry {i} reads cache unit {e.cache} before any entry has written it")
-                a = self.blocks[self.plan[owners[e.cache]].layer].mixer.cache_requirement()
-                b = self.blocks[e.layer].mixer.cache_requirement()
+                a = self.blocks[self.plan[owners[e.cache]].layer].cache_requirement()
+                b = self.blocks[e.layer].cache_requirement()
                 if a != b:
                     raise ValueError(f"plan entry {i} reads cache unit {e.cache}, whose owner keeps something else ({a} vs {b})")
 
     @property
     def graph_safe(self) -> bool:
         """Every part agrees to be replayed from a HIP graph (a block answers for its members)."""
-        parts = [*self.blocks, self.final_norm, self.head]
-        if self.embedding.position is not None:
-            parts.append(self.embedding.position)
-        return all(getattr(p, "graph_safe", False) for p in parts)
+        return all(getattr(p, "graph_safe", False) for p in (self.embedding, *self.blocks, self.final_norm, self.head))
 
     @property
     def max_positions(self) -> Optional[int]:
@@ -103,7 +69,7 @@ class DecoderLm:
 
     def cache_requirements(self) -> List[Tuple[int, object]]:
         """(cache unit, requirement) of every unit that a plan entry writes."""
-        return [(e.cache, self.blocks[e.layer].mixer.cache_requirement()) for e in self.plan if e.writes_cache]
+        return [(e.cache, self.blocks[e.layer].cache_requirement()) for e in self.plan if e.writes_cache]
 
     def forward(self, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
         """Run the step's tokens through the plan; float32 logits ``[len(logit_rows), vocab]``."""

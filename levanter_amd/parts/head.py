@@ -16,14 +16,16 @@ from .spec import PartSpec
 class TiedHead(Head):
     graph_safe = True
 
-    """Uses the embedding's table (set by the decoder with ``tie``); holds no second copy."""
+    """Uses the embedding's table (taken in ``bind``); holds no second copy."""
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
         self.table = None
 
-    def tie(self, table: torch.Tensor) -> None:
-        self.table = table  # [vocab, dim], compute dtype
+    def bind(self, embedding) -> None:
+        if embedding.table is None:
+            raise ValueError("a tied head needs an embedding with a token table")
+        self.table = embedding.table  # [vocab, dim], compute dtype
 
     def __call__(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         logits = ctx.empty(h.shape[0], self.table.shape[0], torch.float32)

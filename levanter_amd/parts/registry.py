@@ -1,5 +1,5 @@
-"""Registries of part kinds. Each family (norm, position encoding, mixer, feed-forward, block,
-head) maps a kind name to a class; a model description names kinds, ``build_part`` constructs
+"""Registries of part kinds. Each family (norm, position encoding, mixer, feed-forward, embedding,
+head, block) maps a kind name to a class; a model description names kinds, ``build_part`` constructs
 them. Registering a new kind needs no change to the framework's files:
 
     @MIXERS.register("my_mixer")
@@ -47,3 +47,24 @@ MIXERS: PartRegistry = PartRegistry("mixer")
 FEED_FORWARDS: PartRegistry = PartRegistry("feed-forward")
 BLOCKS: PartRegistry = PartRegistry("block")
 HEADS: PartRegistry = PartRegistry("head")
+EMBEDDINGS: PartRegistry = PartRegistry("embedding")
+
+FAMILIES: Dict[str, PartRegistry] = {"norm": NORMS, "position": POSITION_ENCODINGS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS,
+                                     "embedding": EMBEDDINGS, "head": HEADS}
+
+
+def part_class(kind: str, family: str = ""):
+    """The class of a part: from its family's registry, or (no family given) from the one registry that knows the kind."""
+    if family:
+        try:
+            return FAMILIES[family].get(kind)
+        except KeyError as e:
+            if family not in FAMILIES:
+                raise KeyError(f"unknown part family {family!r}; families: {', '.join(FAMILIES)}") from None
+            raise e
+    found = [(name, reg) for name, reg in FAMILIES.items() if kind in reg._kinds]
+    if len(found) == 1:
+        return found[0][1].get(kind)
+    if not found:
+        raise KeyError(f"no part family has a kind {kind!r}")
+    raise KeyError(f"the kind {kind!r} exists in several families ({', '.join(n for n, _ in found)}); name the family in the description")

@@ -1,9 +1,12 @@
 """The description of a model as data: what ``models/<architecture>.py`` produces from a
 configuration and what ``parts.decoder`` builds a runnable model from.
 
-A part (norm, position encoding, mixer, feed-forward) is described by its kind (a name in
-that part family's registry), its sizes and constants, and the checkpoint tensor behind each
-of its parameters. A layer names one part of each family and the block that arranges them.
+A part (norm, position encoding, mixer, feed-forward, embedding, head) is described by its
+family, its kind (a name in that family's registry), its sizes and constants, and the
+checkpoint tensor behind each of its parameters. A layer names the block that arranges its
+parts and the parts themselves by the role they play in that block: which roles there are is
+the block's business (the pre-norm block has ``norm1``, ``mixer``, ``norm2``,
+``feed_forward``; a block with parallel branches, four norms or no feed-forward names others).
 The order in which layers run is a list of ``PlanEntry``: it may name a layer twice, and an
 entry may read the cache that another entry writes.
 """
@@ -28,15 +31,33 @@ class PartSpec:
     kind: str
     params: Dict[str, Any] = field(default_factory=dict)
     tensors: Dict[str, TensorSpec] = field(default_factory=dict)
+    family: str = ""
+    """The registry the kind is looked up in: "norm", "mixer", "feed_forward", "position", "embedding" or "head".
+    Empty: the one registry that knows the kind."""
 
 
-@dataclass
 class LayerSpec:
-    block: str
-    norm1: PartSpec
-    mixer: PartSpec
-    norm2: PartSpec
-    feed_forward: PartSpec
+    """``block``: the kind of block; ``parts``: role in that block -> part. Roles read and write like attributes
+    (``layer.mixer``, ``layer.norm1 = ...``)."""
+
+    def __init__(self, block: str, parts: Optional[Dict[str, PartSpec]] = None, **roles: PartSpec):
+        object.__setattr__(self, "block", block)
+        object.__setattr__(self, "parts", {**(parts or {}), **roles})
+
+    def __getattr__(self, role: str) -> PartSpec:
+        try:
+            return object.__getattribute__(self, "parts")[role]
+        except KeyError:
+            raise AttributeError(f"this layer ({self.block}) has no part {role!r}; it has {', '.join(self.parts)}") from None
+
+    def __setattr__(self, role: str, value) -> None:
+        if role == "block":
+            object.__setattr__(self, role, value)
+        else:
+            self.parts[role] = value
+
+    def __repr__(self) -> str:
+        return f"LayerSpec({self.block!r}, {self.parts!r})"
 
 
 @dataclass(frozen=True)
@@ -55,12 +76,12 @@ class ModelSpec:
     vocab_size: int
     dim: int
     embedding: PartSpec
-    """kind "token_embedding": params {position: PartSpec of a position encoding}."""
+    """family "embedding"; kind "token_embedding": params {position: PartSpec of a position encoding}."""
     layers: List[LayerSpec]
     plan: List[PlanEntry]
     final_norm: PartSpec
     head: PartSpec
-    """kind "tied_head" (reads the token table) or "linear_head"."""
+    """family "head"; kind "tied_head" (uses the embedding's table) or "linear_head"."""
     max_positions: Optional[int] = None
     """Largest sequence length the architecture itself allows (a position table's rows)."""
     strip_prefixes: Tuple[str, ...] = ()
@@ -87,7 +108,7 @@ class ModelSpec:
 
         add(self.embedding)
         for layer in self.layers:
-            for part in (layer.norm1, layer.mixer, layer.norm2, layer.feed_forward):
+            for part in layer.parts.values():
                 add(part)
         add(self.final_norm)
         add(self.head)

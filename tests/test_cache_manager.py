@@ -243,11 +243,12 @@ def test_padding_tokens_of_a_replayed_step_beside_a_window_that_has_moved_on():
     positions, token_seq = view(1), view(2)
     assert list(positions[5:]) == [0, 0, 0] and list(token_seq[5:]) == [0, 0, 0]
     for gi, g in enumerate(cache.groups):
-        bt = view(7 + 2 * gi).reshape(b.n_seqs, b.max_blocks)
-        dest = view(8 + 2 * gi)
+        bt = view(8 + 2 * gi).reshape(b.n_seqs, b.max_blocks)
+        dest = view(9 + 2 * gi)
         assert (dest[:5] >= 0).all() and (dest[5:] == -1).all()
         w = g.requirement.window
         for t in range(5):  # real tokens: every visible key has a page
             lo = 0 if w is None else max(0, positions[t] - w + 1)
             assert (bt[token_seq[t], lo // 16: positions[t] // 16 + 1] != NO_PAGE).all()
-    assert view(7 + 2 * 1).reshape(b.n_seqs, b.max_blocks)[0, 0] == NO_PAGE  # what the padding tokens point at
+    assert list(view(7)) == [h.slot for h in handles] + [-1, -1, -1]  # padding tokens belong to no slot
+    assert view(8 + 2 * 1).reshape(b.n_seqs, b.max_blocks)[0, 0] == NO_PAGE  # what the padding tokens point at

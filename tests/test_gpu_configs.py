@@ -41,6 +41,33 @@ def test_a_model_without_biases(dtype):
     check_all_cuttings("no biases", raw, 5, dtype, [70, 45, 100, 37])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_reference_s_schedules_through_trace_run(dtype):
+    """The step schedules of the reference's paged-attention tests (tests/inference/test_paged_attention.py:293-442):
+    two requests filled by [[4,2],[0,1],[0,1],[2,1],[1,2],[1,1]] tokens a step, and a prefix of 1 to 3 tokens followed
+    by four chunks of 1, 2, 3 or 8 tokens of both."""
+    raw, seed = TINY["B"]
+    d = write_model(raw, seed, torch.float32 if dtype == "float32" else torch.bfloat16)
+    weights = read_weights(d)
+    reqs = TR.random_requests(raw["vocab_size"], [35, 35], 21)
+    rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    plain = {rid: P.plain_logits(weights, raw, torch.tensor(t), rounding=rounding) for rid, t in reqs.items()}
+    steps, owner = [], {}
+    schedules = [TR.REFERENCE_RAGGED_SCHEDULE] + [TR.reference_chunk_schedule(p, c) for p in TR.REFERENCE_PREFIX_SIZES
+                                                  for c in TR.REFERENCE_CHUNK_SIZES]
+    for i, schedule in enumerate(schedules):
+        n = sum(a for a, _ in schedule)
+        ids = (f"a{i}", f"b{i}")
+        owner.update({ids[0]: "r0", ids[1]: "r1"})
+        steps += TR.trace_two_requests(reqs["r0"][:n], reqs["r1"][:n], schedule, ids=ids)
+    TR.number(steps)
+    out = run_trace(d, dtype, steps, 128)
+    want = TR.expected_rows(steps, lambda rid: plain[owner[rid]])
+    tol = TOL_F32 if dtype == "float32" else dict(rtol=2e-2, atol=8e-3)
+    for k, w in want.items():
+        torch.testing.assert_close(read_step(out, k, raw["vocab_size"]).double(), w, **tol, msg=lambda m: f"step {k}: {m}")
+
+
 class _LazyLogits:
     """Rows of ``hidden @ table^T`` on demand (a vocabulary of 50,257 makes all rows of a long request too many)."""
 

@@ -522,8 +522,184 @@ def test_a_new_architecture_registers_without_touching_the_framework(tmp_path):
         engine = InferenceEngine.from_pretrained(str(tmp_path), InferenceEngineConfig(max_seqs=2, max_pages_per_seq=4, compute_dtype="float32"))
         res = engine.generate([Request(prompt_tokens=[1, 2, 3], request_id=0, max_new_tokens=5)])
         assert len(res.tokens[0]) == 5
+        # the numbers: every generated token is the argmax of a plain computation whose norms are RMS norms
+        w = read_weights(str(tmp_path))
+        raw = {"n_embd": 48, "n_head": 3, "n_layer": 2, "vocab_size": 300, "n_positions": 64, "activation_function": "gelu_new"}
+
+        def rms(x, weight, bias):
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * weight + bias
+
+        toks = [1, 2, 3] + res.tokens[0]
+        x = P.plain_embed(torch.tensor(toks), torch.arange(len(toks)), w["wte.weight"], w["wpe.weight"])
+        for i in range(2):
+            p = f"h.{i}."
+            x = x + P.plain_attention_layer(rms(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"]), w, p, raw, i)
+            x = x + P.plain_mlp(rms(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"]), w, p, raw)
+        logits = rms(x, w["ln_f.weight"], w["ln_f.bias"]) @ w["wte.weight"].T
+        assert logits[2:-1].argmax(-1).tolist() == res.tokens[0]
+        with_layernorm = P.plain_logits(w, raw, torch.tensor(toks))
+        assert float((with_layernorm - logits).abs().max()) > 1e-2  # the two norms are told apart
+        step_logits = engine.runner.step([__import__("levanter_amd.engine", fromlist=["StepEntry"]).StepEntry(engine.cache.open("z"), toks, list(range(len(toks))))])
+        torch.testing.assert_close(step_logits.cpu().double(), logits, rtol=1e-4, atol=1e-5)
     finally:
         LmConfig.unregister("toy_gpt_rms")
+
+
+def test_other_blocks_and_another_embedding_register_without_touching_the_framework():
+    """Arrangements GPT-2 does not have, defined here: a block whose mixer and feed-forward read the same normed input
+    and add to the residual side by side (three parts: one norm), a block with a norm after each branch as well (six
+    parts), a layer that has a mixer and no feed-forward, and an embedding that scales the token rows. Each is a class
+    registered from this file and named in a description; the framework's files stay as they are."""
+    from levanter_amd.parts import BLOCKS, EMBEDDINGS, Block, LayerSpec, PartSpec, TensorSpec
+    from levanter_amd.parts.embedding import TokenEmbedding
+
+    @BLOCKS.register("toy_parallel")
+    class Parallel(Block):
+        roles = ("norm", "mixer", "feed_forward")
+
+        def forward(self, x, ctx, unit, writes_cache):
+            h = self.parts["norm"](x, ctx)
+            self.parts["mixer"].forward(h, x, ctx, unit, writes_cache)
+            self.parts["feed_forward"].forward(h, x, ctx)
+
+    @BLOCKS.register("toy_sandwich")
+    class Sandwich(Block):
+        roles = ("norm1", "mixer", "post1", "norm2", "feed_forward", "post2")
+
+        def forward(self, x, ctx, unit, writes_cache):
+            p = self.parts
+            for pre, branch, post in (("norm1", "mixer", "post1"), ("norm2", "feed_forward", "post2")):
+                y = torch.zeros_like(x)
+                if branch == "mixer":
+                    p[branch].forward(p[pre](x, ctx), y, ctx, unit, writes_cache)
+                else:
+                    p[branch].forward(p[pre](x, ctx), y, ctx)
+                x += p[post](y, ctx).float()
+
+    @BLOCKS.register("toy_mixer_only")
+    class MixerOnly(Block):
+        roles = ("norm1", "mixer")
+
+        def forward(self, x, ctx, unit, writes_cache):
+            self.parts["mixer"].forward(self.parts["norm1"](x, ctx), x, ctx, unit, writes_cache)
+
+    @EMBEDDINGS.register("toy_scaled_embedding")
+    class Scaled(TokenEmbedding):
+        def __call__(self, ctx):
+            x = super().__call__(ctx)  # token row + position row
+            pos = self.position.embedding_table()[ctx.attention.positions.long()].float()
+            return (x - pos) * float(self.spec.params["multiplier"]) + pos
+
+    try:
+        from levanter_amd.config import LmConfig
+
+        raw = dict(TINY_A, n_layer=3)
+        d = write_model(raw, 2, torch.float32)
+        w = read_weights(d)
+        t32 = {k: v.float() for k, v in w.items()}
+        spec = LmConfig.from_dict(raw).model_spec()
+        l0, l1, l2 = spec.layers
+        spec.layers[0] = LayerSpec("toy_parallel", norm=l0.norm1, mixer=l0.mixer, feed_forward=l0.feed_forward)
+        post = lambda name: PartSpec("layernorm", {"dim": 64, "eps": 1e-5, "bias": True},
+                                     {"weight": TensorSpec(name + ".weight", (64,), init="one_plus_normal"), "bias": TensorSpec(name + ".bias", (64,))})
+        spec.layers[1] = LayerSpec("toy_sandwich", norm1=l1.norm1, mixer=l1.mixer, post1=post("h.0.ln_2"), norm2=l1.norm2,
+                                   feed_forward=l1.feed_forward, post2=post("ln_f"))  # tensors of the file, used a second time
+        spec.layers[2] = LayerSpec("toy_mixer_only", norm1=l2.norm1, mixer=l2.mixer)
+        spec.embedding.kind = "toy_scaled_embedding"
+        spec.embedding.params["multiplier"] = 3.0
+        assert "h.2.mlp.c_fc.weight" not in spec.all_tensors() and "h.0.ln_2.weight" in spec.all_tensors()
+        toks = torch.randint(0, 512, (45,), generator=torch.Generator().manual_seed(12)).tolist()
+        ln = lambda x, name: P.plain_layernorm(x, w[name + ".weight"], w[name + ".bias"], 1e-5)
+        x = 3.0 * w["wte.weight"][torch.tensor(toks)] + w["wpe.weight"][:45]
+        h = ln(x, "h.0.ln_1")
+        x = x + P.plain_attention_layer(h, w, "h.0.", raw, 0) + P.plain_mlp(h, w, "h.0.", raw)
+        x = x + ln(P.plain_attention_layer(ln(x, "h.1.ln_1"), w, "h.1.", raw, 1), "h.0.ln_2")
+        x = x + ln(P.plain_mlp(ln(x, "h.1.ln_2"), w, "h.1.", raw), "ln_f")
+        x = x + P.plain_attention_layer(ln(x, "h.2.ln_1"), w, "h.2.", raw, 2)
+        want = ln(x, "ln_f") @ w["wte.weight"].T
+        for cuts in ([45], [17, 2, 25, 1]):
+            got, cache, _ = _run_cut(spec, t32, "float32", toks, cuts)
+            torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-5)
+        with pytest.raises(ValueError, match="lacks feed_forward"):
+            bad = LmConfig.from_dict(raw).model_spec()
+            bad.layers[0] = LayerSpec("toy_parallel", norm=l0.norm1, mixer=l0.mixer)
+            from levanter_amd.parts import DecoderLm
+            DecoderLm(bad, t32, _env("float32"))
+    finally:
+        for k in ("toy_parallel", "toy_sandwich", "toy_mixer_only"):
+            BLOCKS.unregister(k)
+        EMBEDDINGS.unregister("toy_scaled_embedding")
+
+
+def test_a_toy_state_mixer_that_steers_from_the_device_is_replayed_from_a_graph():
+    """The running-mean mixer again, written with device-side facts only (``ctx.token_slots``, positions, request
+    rows): it declares itself ``graph_safe``, so decode steps of a model that holds it are recorded and replayed,
+    padding tokens and all; their logits equal the eager runner's."""
+    from levanter_amd.cache import SlotState
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import make_cache
+    from levanter_amd.parts import MIXERS, DecoderLm, Mixer, PartSpec
+
+    D = 64
+
+    @MIXERS.register("toy_running_mean_on_device")
+    class RunningMean(Mixer):
+        graph_safe = True
+
+        def cache_requirement(self):
+            return SlotState((D + 1,), "float32")
+
+        def forward(self, h, x, ctx, unit, writes_cache):
+            pos, seq, slots = ctx.attention.positions, ctx.attention.token_seq, ctx.token_slots
+            valid = slots >= 0
+            slot = slots.clamp(min=0).long()
+            earlier = (seq[:, None] == seq[None, :]) & (pos[None, :] <= pos[:, None]) & valid[None, :] & valid[:, None]
+            hf = h.float()
+            sums = unit.state[slot, :D] + earlier.float() @ hf
+            x += 0.5 * sums / (pos + 1).float()[:, None]
+            unit.state.index_add_(0, slot, torch.cat([hf, torch.ones_like(hf[:, :1])], 1) * valid[:, None].float())
+
+    try:
+        d = write_model(TINY_A, 0, torch.float32)
+        w = read_weights(d)
+        t32 = {k: v.float() for k, v in w.items()}
+        spec = _toy_spec(mixers=[None, PartSpec("toy_running_mean_on_device", {}, {})])
+        env = _env("float32")
+        model = DecoderLm(spec, t32, env)
+        assert model.graph_safe
+        cfg = InferenceEngineConfig(max_pages=32, max_seqs=8, page_size=16, max_pages_per_seq=8, compute_dtype="float32")
+        gen = torch.Generator().manual_seed(14)
+        seqs = [torch.randint(0, 512, (n,), generator=gen).tolist() for n in (50, 40, 45, 38, 47)]
+
+        def plain(toks):
+            n = len(toks)
+            x = P.plain_embed(torch.tensor(toks), torch.arange(n), w["wte.weight"], w["wpe.weight"])
+            x = P.plain_block(x, w, TINY_A, 0)
+            hh = P.plain_layernorm(x, w["h.1.ln_1.weight"], w["h.1.ln_1.bias"], 1e-5)
+            x = x + 0.5 * torch.cumsum(hh, 0) / torch.arange(1, n + 1).unsqueeze(1)
+            x = x + P.plain_mlp(P.plain_layernorm(x, w["h.1.ln_2.weight"], w["h.1.ln_2.bias"], 1e-5), w, "h.1.", TINY_A)
+            return P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5) @ w["wte.weight"].T
+
+        want = [plain(t) for t in seqs]
+        cache = make_cache(model, cfg)
+        runner = ModelRunner(model, cache, env)
+        assert runner.use_graphs
+        handles = [cache.open(i) for i in range(5)]
+        got = runner.step([StepEntry(h, seqs[i][:10 + i], list(range(10 + i))) for i, h in enumerate(handles)]).cpu()
+        r0 = 0
+        for i in range(5):
+            torch.testing.assert_close(got[r0:r0 + 10 + i].double(), want[i][:10 + i], rtol=1e-4, atol=1e-4)
+            r0 += 10 + i
+        for step in range(24):  # five single tokens, filled up to eight: replayed from the second step on
+            got = runner.step([StepEntry(h, [seqs[i][h.length]], [0]) for i, h in enumerate(handles)]).cpu()
+            for i, h in enumerate(handles):
+                torch.testing.assert_close(got[i].double(), want[i][h.length - 1], rtol=1e-4, atol=1e-4)
+        assert any(not isinstance(v, str) for v in runner._graphs.values())
+        for i, h in enumerate(handles):
+            assert float(cache.state.tensors[1][h.slot, D]) == h.length  # padding tokens were not counted
+    finally:
+        MIXERS.unregister("toy_running_mean_on_device")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -28,12 +28,22 @@ def setup(request):
     return raw, model, env, reqs, plain
 
 
-def replay(model, env, steps, max_tokens):
+def replay(model, env, steps, max_tokens, slots=None):
+    """``slots``: request id -> the slot it must occupy."""
     ps = 16
     cfg = InferenceEngineConfig(max_pages=max_tokens // ps, max_seqs=4, page_size=ps, max_pages_per_seq=16, compute_dtype="float32")
     cache = make_cache(model, cfg)
     runner = ModelRunner(model, cache, env)
     live, out = {}, {}
+    if slots:  # a fresh manager hands out slots 0, 1, 2 ... in order
+        who = {slot: rid for rid, slot in slots.items()}
+        opened = [cache.open(who.get(i, ("placeholder", i))) for i in range(max(who) + 1)]
+        for h in opened:
+            if h.request_id in slots:
+                live[h.request_id] = h
+            else:
+                cache.close(h)
+        assert {rid: live[rid].slot for rid in slots} == slots
     for s in steps:
         entries = []
         for e in s["entries"]:
@@ -156,3 +166,30 @@ def test_a_step_that_fails_in_the_model_gives_its_pages_back(setup, monkeypatch)
     cache.close(a)
     cache.close(b)
     assert all(g.pool.n_free == g.pool.n_pages for g in cache.groups)
+
+
+def test_the_reference_s_ragged_schedule(setup):
+    """tests/inference/test_paged_attention.py:378-442: two requests of 8 tokens filled by [[4,2],[0,1],[0,1],[2,1],[1,2],[1,1]]
+    tokens a step (a request is left out where its count is 0); every step's rows equal the whole sequence's."""
+    raw, model, env, reqs, plain = setup
+    t0, t1 = reqs["r0"][:8], reqs["r1"][:8]
+    steps = TR.trace_two_requests(t0, t1, TR.REFERENCE_RAGGED_SCHEDULE)
+    got = replay(model, env, steps, 128)
+    want = TR.expected_rows(steps, lambda rid: plain["r0" if rid == "a" else "r1"])
+    for k in want:
+        torch.testing.assert_close(got[k].double(), want[k], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("slots", TR.REFERENCE_SLOT_ORDERS)
+@pytest.mark.parametrize("chunk", TR.REFERENCE_CHUNK_SIZES)
+def test_the_reference_s_chunked_prefill_in_every_slot_order(setup, slots, chunk):
+    """tests/inference/test_paged_attention.py:293-376: a prefix of 1, 2 or 3 tokens of two requests, then four chunks of
+    1, 2, 3 or 8 tokens each, with the requests in slots [0,1], [1,0], [2,0], [0,2], [2,1]."""
+    raw, model, env, reqs, plain = setup
+    for prefix in TR.REFERENCE_PREFIX_SIZES:
+        n = prefix + 4 * chunk
+        steps = TR.trace_two_requests(reqs["r0"][:n], reqs["r1"][:n], TR.reference_chunk_schedule(prefix, chunk))
+        got = replay(model, env, steps, 128, slots={"a": slots[0], "b": slots[1]})
+        want = TR.expected_rows(steps, lambda rid: plain["r0" if rid == "a" else "r1"])
+        for k in want:
+            torch.testing.assert_close(got[k].double(), want[k], rtol=1e-4, atol=1e-5)

@@ -134,3 +134,30 @@ def expected_rows(steps, plain_logits_of):
 
 def to_jsonl(steps) -> str:
     return "".join(json.dumps(s) + "\n" for s in steps)
+
+
+# ---- the schedules of the reference's own paged-attention tests (tests/inference/test_paged_attention.py:293-442) ----
+REFERENCE_RAGGED_SCHEDULE = [[4, 2], [0, 1], [0, 1], [2, 1], [1, 2], [1, 1]]  # tokens of request 0 and 1 in each step
+REFERENCE_SLOT_ORDERS = [[0, 1], [1, 0], [2, 0], [0, 2], [2, 1]]              # the slots the two requests occupy
+REFERENCE_PREFIX_SIZES = [1, 2, 3]
+REFERENCE_CHUNK_SIZES = [1, 2, 3, 8]
+
+
+def trace_two_requests(tokens0, tokens1, schedule, ids=("a", "b")):
+    """Steps that bring ``schedule[i] = [n0, n1]`` tokens of two requests (0: the request is left out of the step)."""
+    steps, off = [], [0, 0]
+    toks = (tokens0, tokens1)
+    for sizes in schedule:
+        entries = []
+        for r in (0, 1):
+            if sizes[r]:
+                entries.append(_entry(ids[r], toks[r], off[r], sizes[r]))
+                off[r] += sizes[r]
+        steps.append({"entries": entries, "end": [ids[r] for r in (0, 1) if sizes[r] and off[r] == len(toks[r])]})
+    assert off == [len(tokens0), len(tokens1)]
+    return number(steps)
+
+
+def reference_chunk_schedule(prefix, chunk):
+    """A prefix of both requests in one step, then four chunks each, as the reference's chunked-prefill test does."""
+    return [[prefix, prefix]] + [[chunk, chunk]] * 4
