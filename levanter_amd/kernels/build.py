@@ -2,6 +2,7 @@
 
 * ``core``: errors, embedding / norms / KV write / sampling, the 32-bit GEMM and attention;
 * ``gemm_mfma``: the bfloat16 GEMMs on the matrix cores;
+* ``gemm_library``: the vendor library's GEMM (hipBLASLt) for prompt-sized row counts, where it is ahead;
 * ``attn_hd<N>``: the bfloat16 attention on the matrix cores for head size N (16 .. 128 in steps of 16).
 
 A model loads ``core`` and, in bfloat16, ``gemm_mfma`` and the attention unit of its own head size, so a first
@@ -38,7 +39,10 @@ UNITS: Dict[str, List[Tuple[str, List[str], str]]] = {
         ("attention_common.hip", [], "attention_common.o"),
     ],
     "gemm_mfma": [("gemm_mfma.hip", [], "gemm_mfma.o")],
+    "gemm_library": [("gemm_library.hip", [], "gemm_library.o")],
 }
+# libraries a unit is linked against
+UNIT_LINK_FLAGS: Dict[str, List[str]] = {"gemm_library": ["-lhipblaslt"]}
 for _hd in MFMA_ATTENTION_HEAD_DIMS:
     UNITS[f"attn_hd{_hd}"] = [
         ("attention_mfma.hip", [f"-DLEV_HD={_hd}"], f"attention_mfma_hd{_hd}.o"),
@@ -105,6 +109,7 @@ def source_hash(unit: str = "core") -> str:
             h.update(f.read())
     for _, defines, obj in UNITS[unit]:
         h.update((" ".join(defines) + obj).encode())
+    h.update(" ".join(UNIT_LINK_FLAGS.get(unit, [])).encode())
     return h.hexdigest()[:16]
 
 
@@ -185,7 +190,8 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
         lib = paths[u]
         objs = [os.path.join(obj_dir, obj_name) for _, _, obj_name in UNITS[u]]
         tmp = lib + f".tmp{os.getpid()}"
-        r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], capture_output=True, text=True, env=env)
+        r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs, *UNIT_LINK_FLAGS.get(u, [])],
+                           capture_output=True, text=True, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed to link {lib_name(u)}:\n{_filter(r.stderr)}")
         os.replace(tmp, lib)

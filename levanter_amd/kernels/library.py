@@ -84,6 +84,9 @@ class HipKernels:
             "lev_attention_mfma_workspace": [c_int] * 5,
         })
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
+        # the vendor library's GEMM for prompt-sized row counts (see use_library); "0" keeps every product on our kernels
+        self.gemm_library = os.environ.get("LEVANTER_AMD_GEMM_LIBRARY", "1") != "0"
+        self._library_refused = set()
         self._sample_ws = None
         self._units = {}
         self._ws, self._ws_outgrown, self._ws_need = {}, [], {}  # GEMM scratch memory per device, see _workspace
@@ -106,7 +109,13 @@ class HipKernels:
                 lib = ctypes.CDLL(path)
             except OSError as e:
                 raise KernelError(f"the HIP library {path} cannot be loaded: {e}") from None
-            if unit == "gemm_mfma":
+            if unit == "gemm_library":
+                self._set_signatures(lib, {
+                    "lev_linear_library": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long]
+                    + [c_int] * 5 + [c_void_p],
+                    "lev_linear_library_workspace": [],
+                })
+            elif unit == "gemm_mfma":
                 self._set_signatures(lib, {
                     "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p]
                     + [c_int] * 5 + [c_void_p],
@@ -201,6 +210,20 @@ class HipKernels:
             ldr = ldo if residual is out else _rows(residual, "linear: residual")
         act = ACTIVATIONS[activation]
         if adt == torch.bfloat16 and self.use_mfma and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0:
+            if self.gemm_library and self.use_library(M, N, K, act):
+                key = (M, N, K, act, bias is None, residual is None, odt)
+                # never while a HIP graph is being recorded: what the library records besides its kernel is not ours to vouch for
+                if key not in self._library_refused and not torch.cuda.is_current_stream_capturing():
+                    lib = self._unit("gemm_library")
+                    need = lib.lev_linear_library_workspace()
+                    ws = self._workspace(need, a.device)
+                    rc = lib.lev_linear_library(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws), need,
+                                                M, N, K, act, _DT[odt], _stream())
+                    if rc == 0:
+                        return
+                    if rc < 0:
+                        self._check(rc)
+                    self._library_refused.add(key)  # the library has no kernel for it: ours from now on
             gemm = self._unit("gemm_mfma")
             need = self._ws_need.get((M, N, K))
             if need is None:  # partial sums of a K range split over workgroups
@@ -211,6 +234,20 @@ class HipKernels:
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
                                                    M, N, K, act, _DT[adt], _DT[odt], _stream()))
+
+    LIBRARY_ACTIVATIONS = (ACTIVATIONS["none"], ACTIVATIONS["gelu_new"], ACTIVATIONS["relu"])
+    LIBRARY_MIN_ROWS = 256
+
+    @classmethod
+    def use_library(cls, M: int, N: int, K: int, act: int) -> bool:
+        """Which products go to the vendor library: prompt-sized row counts with an epilogue the library has. Measured
+        on MI355X at the widths of GPT-2 7B and XL (see gemm_library.hip): ours are ahead up to a few hundred rows and
+        on narrow outputs of long sums (K >= 4 N) below a thousand rows."""
+        if act not in cls.LIBRARY_ACTIVATIONS or M < cls.LIBRARY_MIN_ROWS:
+            return False
+        if M < 320 and N * K < (1 << 24):  # weights of a few MB: ours up to 320 rows
+            return False
+        return not (K >= 4 * N and M < 1024)
 
     # ---- cache write -----------------------------------------------------------------------
     def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int) -> None:

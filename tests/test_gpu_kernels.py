@@ -202,6 +202,65 @@ def test_linear_bf16_large_weights_at_20_to_128_rows(K, M, K_, N):
     assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-3
 
 
+@pytest.mark.parametrize("library", [True, False])
+@pytest.mark.parametrize("M,K_,N", [(256, 4096, 4096), (300, 1600, 6400), (1000, 2048, 6151), (2048, 4096, 1608), (1024, 6400, 1600),
+                                    (513, 1024, 50257)])
+def test_linear_bf16_prompt_sized_rows_with_and_without_the_vendor_library(K, library, M, K_, N, monkeypatch):
+    """From 256 rows the bfloat16 product goes to the vendor library where that is ahead (``use_library``), with the
+    epilogues it has; ``gemm_library = False`` keeps it on the tile kernel. Both against the float64 statement, with
+    every epilogue, both output types, a row stride above K and widths that are no multiple of 16."""
+    monkeypatch.setattr(K, "gemm_library", library)
+    monkeypatch.setattr(K, "use_library", lambda M, N, K_, act: act in K.LIBRARY_ACTIVATIONS)  # every shape of this test
+    calls = []
+    if library:
+        lib = K._unit("gemm_library")
+        real = lib.lev_linear_library
+        monkeypatch.setattr(K._units["gemm_library"], "lev_linear_library", lambda *a: calls.append(real(*a)) or calls[-1])
+    lda = K_ + 8
+    a = _rand(M, lda, dtype=torch.bfloat16, seed=M).to(DEV)[:, :K_]
+    w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=N).to(DEV)
+    bias = _rand(N, seed=3).to(DEV)
+    base = a.double() @ w.double().t()
+    gelu_tanh = lambda u: torch.nn.functional.gelu(u, approximate="tanh")
+    # float32 output with bias and residual, in place and from another tensor
+    out = _rand(M, N, seed=4).to(DEV)
+    want = base + bias.double() + out.double()
+    K.linear(a, w, bias, out, residual=out)
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-3
+    res = _rand(M, N, seed=5).to(DEV)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    K.linear(a, w, None, out, residual=res)
+    assert float((out.double() - (base + res.double())).abs().max() / want.abs().max()) < 2e-3
+    # bfloat16 output with bias and the tanh GELU; float32 output tells the tanh GELU from the exact one (they differ by 5e-4)
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K.linear(a, w, bias, out, activation="gelu_new")
+    want = gelu_tanh(base + bias.double())
+    assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-2
+    out = torch.full((M, N), float("nan"), device=DEV)
+    K.linear(a * 2, w, None, out, activation="gelu_new")
+    want = gelu_tanh(2 * base)
+    assert float((out.double() - want).abs().max()) < 1e-4 < float((torch.nn.functional.gelu(2 * base) - want).abs().max())
+    # relu without bias, plain with bias, and an activation the library does not have
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K.linear(a, w, None, out, activation="relu")
+    assert float((out.double() - torch.relu(base)).abs().max() / base.abs().max()) < 2e-2
+    K.linear(a, w, bias, out)
+    assert float((out.double() - (base + bias.double())).abs().max() / base.abs().max()) < 2e-2
+    n_library = len(calls)
+    K.linear(a, w, bias, out, activation="silu")
+    assert float((out.double() - torch.nn.functional.silu(base + bias.double())).abs().max() / base.abs().max()) < 2e-2
+    if library:
+        assert n_library == 6 and len(calls) == 6 and all(rc == 0 for rc in calls), calls  # the library took all but the last
+
+
+def test_which_products_go_to_the_vendor_library(K):
+    none, gelu, silu = 0, 1, 4
+    assert not K.use_library(255, 12288, 4096, none) and K.use_library(256, 12288, 4096, none)
+    assert K.use_library(2048, 16384, 4096, gelu) and not K.use_library(2048, 16384, 4096, silu)
+    assert not K.use_library(512, 4096, 16384, none) and K.use_library(1024, 4096, 16384, none)  # long sums into a narrow output
+    assert not K.use_library(256, 4800, 1600, none) and K.use_library(320, 4800, 1600, none)  # small weights
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_strided_input_and_all_activations(K, dtype):
     M, K_, N = 9, 96, 40
