@@ -65,13 +65,19 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, floa
   *reinterpret_cast<uint2*>(p) = v;
 }
 
+// partial != null: the row is first brought up to date. A matrix product that split its sum into S ranges has left
+// them in partial [S][M][D] instead of adding them to x (its residual); here x[row] += (partial[0] + .. + partial[S-1]
+// + lin_bias), in that order, is stored back and normalised in the same pass: one kernel where a reduction kernel and a
+// norm kernel would each read and write the row.
 template <typename TO, int NT, int NV>
 __global__ void __launch_bounds__(NT)
-norm_reg_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ out,
-                const int* __restrict__ rows, int D, float eps, int rms) {
+norm_reg_kernel(float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ out,
+                const int* __restrict__ rows, int D, float eps, int rms, const float* __restrict__ partial, int S,
+                size_t partial_stride, const float* __restrict__ lin_bias) {
   __shared__ float red[NT / 64];
   const int r = blockIdx.x;
-  const float* xr = x + (size_t)(rows ? rows[r] : r) * D;
+  const size_t row = (size_t)(rows ? rows[r] : r);
+  float* xr = x + row * D;
   // the row, and scale and shift with it: their latency passes during the two reductions
   float4 v[NV], wv[NV], bv[NV];
 #pragma unroll
@@ -81,6 +87,36 @@ norm_reg_kernel(const float* __restrict__ x, const float* __restrict__ w, const 
     v[i] = ok ? *reinterpret_cast<const float4*>(xr + d) : make_float4(0.f, 0.f, 0.f, 0.f);
     wv[i] = ok ? *reinterpret_cast<const float4*>(w + d) : make_float4(0.f, 0.f, 0.f, 0.f);
     bv[i] = ok && b ? *reinterpret_cast<const float4*>(b + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  if (partial) {
+    const float* pr = partial + row * D;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int d = (threadIdx.x + i * NT) * 4;
+      if (d < D) {
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        int s = 0;
+        for (; s + 4 <= S; s += 4) {  // four ranges requested at once, added in their order
+          float4 p[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) p[j] = *reinterpret_cast<const float4*>(pr + (size_t)(s + j) * partial_stride + d);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            t.x += p[j].x; t.y += p[j].y; t.z += p[j].z; t.w += p[j].w;
+          }
+        }
+        for (; s < S; ++s) {
+          const float4 p = *reinterpret_cast<const float4*>(pr + (size_t)s * partial_stride + d);
+          t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+        }
+        if (lin_bias) {
+          const float4 lb = *reinterpret_cast<const float4*>(lin_bias + d);
+          t.x += lb.x; t.y += lb.y; t.z += lb.z; t.w += lb.w;
+        }
+        v[i].x = t.x + v[i].x; v[i].y = t.y + v[i].y; v[i].z = t.z + v[i].z; v[i].w = t.w + v[i].w;
+        *reinterpret_cast<float4*>(xr + d) = v[i];
+      }
+    }
   }
   float mean = 0.f;
   if (!rms) {
@@ -137,19 +173,32 @@ __global__ void norm_kernel(const float* __restrict__ x, const float* __restrict
   }
 }
 
+// Returns false if a pending sum (partial != null) cannot be folded in at this width and alignment: the caller then
+// runs the reduction by itself first.
 template <typename TO>
-static void launch_norm(const float* x, const float* w, const float* b, TO* out, const int* rows, int n_rows, int D, float eps,
-                        int rms, hipStream_t stream) {
+static bool launch_norm(float* x, const float* w, const float* b, TO* out, const int* rows, int n_rows, int D, float eps,
+                        int rms, const float* partial, int S, size_t partial_stride, const float* lin_bias, hipStream_t stream) {
   // rows in registers as vectors of 4: needs D % 4 == 0 and 16-byte aligned pointers
-  const bool vec = (D & 3) == 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)out) & 15) == 0;
-  if (vec && D <= 256 * 4 * 2)
-    norm_reg_kernel<TO, 256, 2><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+  const bool vec = (D & 3) == 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)out | (uintptr_t)partial |
+                                     (uintptr_t)lin_bias) & 15) == 0 && (partial_stride & 3) == 0;
+  // With ranges to add, a row is S + 1 times as many bytes and there are few rows (a decode batch): 1,024 threads a row,
+  // every load of the row and its ranges in flight at once (with 256 threads 64 workgroups took longer over 17 MB of
+  // ranges than the reduction kernel and the norm kernel together).
+  if (partial && vec && D <= 1024 * 4)
+    norm_reg_kernel<TO, 1024, 1><<<n_rows, 1024, 0, stream>>>(x, w, b, out, rows, D, eps, rms, partial, S, partial_stride, lin_bias);
+  else if (partial && vec && D <= 1024 * 4 * 2)
+    norm_reg_kernel<TO, 1024, 2><<<n_rows, 1024, 0, stream>>>(x, w, b, out, rows, D, eps, rms, partial, S, partial_stride, lin_bias);
+  else if (vec && D <= 256 * 4 * 2)
+    norm_reg_kernel<TO, 256, 2><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms, partial, S, partial_stride, lin_bias);
   else if (vec && D <= 256 * 4 * 4)
-    norm_reg_kernel<TO, 256, 4><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+    norm_reg_kernel<TO, 256, 4><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms, partial, S, partial_stride, lin_bias);
   else if (vec && D <= 256 * 4 * 8)
-    norm_reg_kernel<TO, 256, 8><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+    norm_reg_kernel<TO, 256, 8><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms, partial, S, partial_stride, lin_bias);
+  else if (partial)
+    return false;
   else
     norm_kernel<TO, 256><<<n_rows, 256, 0, stream>>>(x, w, b, out, rows, D, eps, rms);
+  return true;
 }
 
 extern "C" int lev_norm(const float* x, const float* w, const float* b, void* out, const int* rows, int n_rows, int D,
@@ -159,9 +208,27 @@ extern "C" int lev_norm(const float* x, const float* w, const float* b, void* ou
   LEV_REQUIRE(eps > 0.f, "norm: eps must be positive");
   if (n_rows == 0) return 0;
   if (out_dtype == LEV_F32)
-    launch_norm<float>(x, w, b, (float*)out, rows, n_rows, D, eps, rms, stream);
+    launch_norm<float>(const_cast<float*>(x), w, b, (float*)out, rows, n_rows, D, eps, rms, nullptr, 0, 0, nullptr, stream);
   else
-    launch_norm<bf16_t>(x, w, b, (bf16_t*)out, rows, n_rows, D, eps, rms, stream);
+    launch_norm<bf16_t>(const_cast<float*>(x), w, b, (bf16_t*)out, rows, n_rows, D, eps, rms, nullptr, 0, 0, nullptr, stream);
+  return lev_check_launch("norm");
+}
+
+// The norm of rows that a matrix product has not finished yet: x [M][D] += partial[0] + .. + partial[S-1] + lin_bias for the
+// rows that are normalised (all M, or rows[0 .. n_rows)), stored back, then the norm as in lev_norm. Returns 1, with
+// nothing launched, if this width or alignment has no such kernel.
+extern "C" int lev_norm_pending(float* x, const float* partial, int S, const float* lin_bias, const float* w, const float* b,
+                                void* out, const int* rows, int n_rows, int M, int D, float eps, int rms, int out_dtype,
+                                hipStream_t stream) {
+  LEV_REQUIRE(n_rows >= 0 && D > 0 && M > 0 && S >= 1 && partial, "norm: bad sizes rows=%d D=%d M=%d ranges=%d", n_rows, D, M, S);
+  LEV_REQUIRE(out_dtype == LEV_F32 || out_dtype == LEV_BF16, "norm: unknown output dtype %d", out_dtype);
+  LEV_REQUIRE(eps > 0.f, "norm: eps must be positive");
+  if (n_rows == 0) return 0;
+  const size_t stride = (size_t)M * D;
+  const bool ok = out_dtype == LEV_F32
+                      ? launch_norm<float>(x, w, b, (float*)out, rows, n_rows, D, eps, rms, partial, S, stride, lin_bias, stream)
+                      : launch_norm<bf16_t>(x, w, b, (bf16_t*)out, rows, n_rows, D, eps, rms, partial, S, stride, lin_bias, stream);
+  if (!ok) return 1;
   return lev_check_launch("norm");
 }
 

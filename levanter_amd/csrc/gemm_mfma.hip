@@ -302,7 +302,7 @@ static int launch_splitk_reduce(const float* workspace, const float* bias, const
 
 template <typename TO, int BM, int BN>
 static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
-                       long ldo, float* workspace, int M, int N, int K, int act, int S, hipStream_t stream) {
+                       long ldo, float* workspace, int M, int N, int K, int act, int S, int defer, hipStream_t stream) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds_ops = (size_t)2 * (BM + BN) * LDS_STRIDE * sizeof(bf16_t);
   const size_t lds_out = (size_t)4 * 32 * (BN / 2 + 4) * sizeof(float);
@@ -323,6 +323,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
                                                                                    workspace);
   if (S > 1) {
     if (int rc = lev_check_launch("linear_tile")) return rc;
+    if (defer) return 0;  // the caller folds the sum of the ranges into its next kernel
     return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
   }
   return 0;
@@ -802,15 +803,30 @@ static bool use_skinny(int M, int N, int K) {
   return !(M >= 20 && (double)N * K * 2.0 >= 64e6);
 }
 
+// Into how many ranges the sum over K is split (1: the kernel finishes its outputs itself).
+extern "C" int lev_linear_mfma_ranges(int M, int N, int K) {
+  if (use_skinny(M, N, K)) return 1;
+  return M <= 128 ? plan_stream(M, N, K).splits : plan_tiles(M, N, K).splits;
+}
+
 extern "C" long lev_linear_mfma_workspace(int M, int N, int K) {
-  if (use_skinny(M, N, K)) return 0;
-  const int S = M <= 128 ? plan_stream(M, N, K).splits : plan_tiles(M, N, K).splits;
+  const int S = lev_linear_mfma_ranges(M, N, K);
   return S > 1 ? (long)S * M * N * (long)sizeof(float) : 0;
+}
+
+// out = act(sum of the S ranges in workspace [S][M][N] + bias) + residual: what lev_linear_mfma runs itself unless it was
+// asked to leave the ranges to the caller.
+extern "C" int lev_linear_mfma_finish(const float* workspace, const float* bias, const float* residual, long ldr, void* out, long ldo,
+                                      int M, int N, int S, int act, int out_dtype, hipStream_t stream) {
+  LEV_REQUIRE(workspace && M > 0 && N > 0 && S > 1, "linear: nothing to finish (M=%d N=%d ranges=%d)", M, N, S);
+  if (out_dtype == LEV_F32) return launch_splitk_reduce<float>(workspace, bias, residual, ldr, (float*)out, ldo, M, N, S, act, stream);
+  if (out_dtype == LEV_BF16) return launch_splitk_reduce<bf16_t>(workspace, bias, residual, ldr, (bf16_t*)out, ldo, M, N, S, act, stream);
+  return lev_fail("linear: unknown output dtype %d", out_dtype);
 }
 
 template <typename TO>
 static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr, TO* out,
-                         long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
+                         long ldo, float* workspace, int M, int N, int K, int act, int defer, hipStream_t stream) {
   if ((size_t)M * lda >= (1ull << 32)) return lev_fail("linear: the activation matrix is too large (M=%d lda=%ld)", M, lda);
   const StreamPlan plan = plan_stream(M, N, K);
   const int S = plan.splits;
@@ -835,40 +851,43 @@ static int launch_stream(const bf16_t* a, long lda, const bf16_t* w, const float
 #undef LEV_STREAM_MT
 #undef LEV_STREAM
   if (int rc = lev_check_launch("linear_stream")) return rc;
-  if (S > 1) return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
+  if (S > 1 && !defer) return launch_splitk_reduce<TO>(workspace, bias, residual, ldr, out, ldo, M, N, S, act, stream);
   return 0;
 }
 
 template <typename TO>
 static int linear_mfma_typed(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
-                             TO* out, long ldo, float* workspace, int M, int N, int K, int act, hipStream_t stream) {
+                             TO* out, long ldo, float* workspace, int M, int N, int K, int act, int defer, hipStream_t stream) {
   if (use_skinny(M, N, K)) {
     launch_skinny<TO>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act, stream);
   } else if (M <= 128) {
-    return launch_stream<TO>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, stream);
+    return launch_stream<TO>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, defer, stream);
   } else {
     if ((size_t)M * lda >= (1ull << 31) || (size_t)N * K >= (1ull << 31))
       return lev_fail("linear: operands of more than 2^31 elements are not supported (M=%d lda=%ld N=%d K=%d)", M, lda, N, K);
     const TilePlan plan = plan_tiles(M, N, K);
     int rc;
     if (plan.shape == 0)
-      rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+      rc = launch_tile<TO, 256, 256>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, defer, stream);
     else if (plan.shape == 1)
-      rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+      rc = launch_tile<TO, 256, 192>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, defer, stream);
     else if (plan.shape == 2)
-      rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+      rc = launch_tile<TO, 256, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, defer, stream);
     else if (plan.shape == 3)
-      rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+      rc = launch_tile<TO, 128, 128>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, defer, stream);
     else
-      rc = launch_tile<TO, 128, 64>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, stream);
+      rc = launch_tile<TO, 128, 64>(a, lda, w, bias, residual, ldr, out, ldo, workspace, M, N, K, act, plan.splits, defer, stream);
     if (rc) return rc;
   }
   return lev_check_launch("linear_mfma");
 }
 
+// leave_ranges: where the sum over K is split into ranges (lev_linear_mfma_ranges > 1) the kernel stops after writing
+// them to workspace [S][M][N]; bias, activation and residual are then the caller's to apply (lev_linear_mfma_finish, or
+// a kernel of its own that reads the ranges).
 extern "C" int lev_linear_mfma(const void* a, long lda, const void* w, const float* bias, const float* residual, long ldr,
                                void* out, long ldo, void* workspace, int M, int N, int K, int act, int out_dtype,
-                               hipStream_t stream) {
+                               int leave_ranges, hipStream_t stream) {
   LEV_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   LEV_REQUIRE(K % 8 == 0 && lda % 8 == 0, "linear (bfloat16): K=%d and the row stride %ld must be multiples of 8", K, lda);
   LEV_REQUIRE(((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0, "linear (bfloat16): operands must be 16-byte aligned");
@@ -878,9 +897,9 @@ extern "C" int lev_linear_mfma(const void* a, long lda, const void* w, const flo
   if (M == 0) return 0;
   if (out_dtype == LEV_F32)
     return linear_mfma_typed<float>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (float*)out, ldo,
-                                    (float*)workspace, M, N, K, act, stream);
+                                    (float*)workspace, M, N, K, act, leave_ranges, stream);
   if (out_dtype == LEV_BF16)
     return linear_mfma_typed<bf16_t>((const bf16_t*)a, lda, (const bf16_t*)w, bias, residual, ldr, (bf16_t*)out, ldo,
-                                     (float*)workspace, M, N, K, act, stream);
+                                     (float*)workspace, M, N, K, act, leave_ranges, stream);
   return lev_fail("linear: unknown output dtype %d", out_dtype);
 }

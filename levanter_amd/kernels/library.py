@@ -28,6 +28,18 @@ class KernelError(RuntimeError):
     pass
 
 
+class PendingSum:
+    """A matrix product whose sum over K was split into ranges and not finished: ``out`` (float32 ``[M, N]``, the
+    product's residual, updated in place) still lacks ``ranges[0] + .. + ranges[S-1] + bias``. ``HipKernels.norm`` folds
+    that into the norm of ``out``; ``HipKernels.finish`` runs it by itself. Nothing else may read ``out`` or launch
+    another product (the ranges live in the library's one workspace) before one of the two has happened."""
+
+    __slots__ = ("out", "workspace", "n_ranges", "bias", "ldo")
+
+    def __init__(self, out, workspace, n_ranges, bias, ldo):
+        self.out, self.workspace, self.n_ranges, self.bias, self.ldo = out, workspace, n_ranges, bias, ldo
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else c_void_p(t.data_ptr())
 
@@ -75,6 +87,7 @@ class HipKernels:
         self._set_signatures(L, {
             "lev_embed": [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p],
             "lev_norm": [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_int, c_void_p],
+            "lev_norm_pending": [c_void_p, c_void_p, c_int] + [c_void_p] * 5 + [c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
             "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
             "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
             "lev_sample_workspace": [c_int],
@@ -87,6 +100,9 @@ class HipKernels:
         # the vendor library's GEMM for prompt-sized row counts (see use_library); "0" keeps every product on our kernels
         self.gemm_library = os.environ.get("LEVANTER_AMD_GEMM_LIBRARY", "1") != "0"
         self._library_refused = set()
+        # The library's product may be recorded into HIP graphs: replays with changed inputs and eager work between them
+        # give the eager results bit for bit (tests/test_gpu_kernels.py records and replays it at four shapes).
+        self.library_in_graphs = True
         self._sample_ws = None
         self._units = {}
         self._ws, self._ws_outgrown, self._ws_need = {}, [], {}  # GEMM scratch memory per device, see _workspace
@@ -118,8 +134,10 @@ class HipKernels:
             elif unit == "gemm_mfma":
                 self._set_signatures(lib, {
                     "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p]
-                    + [c_int] * 5 + [c_void_p],
+                    + [c_int] * 6 + [c_void_p],
                     "lev_linear_mfma_workspace": [c_int, c_int, c_int],
+                    "lev_linear_mfma_ranges": [c_int, c_int, c_int],
+                    "lev_linear_mfma_finish": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 5 + [c_void_p],
                 })
             else:
                 self._set_signatures(lib, {
@@ -152,8 +170,10 @@ class HipKernels:
                                        _DT[table.dtype], _stream()))
 
     # ---- norms ---------------------------------------------------------------------------
-    def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False) -> None:
-        """LayerNorm (or RMSNorm) of float32 rows into ``out`` (compute dtype). rows: int32 row indices into x."""
+    def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False, pending: Optional[PendingSum] = None) -> None:
+        """LayerNorm (or RMSNorm) of float32 rows into ``out`` (compute dtype). rows: int32 row indices into x.
+        ``pending``: an unfinished product into ``x`` (see ``PendingSum``); its ranges are added to the rows that are
+        normalised, stored back into ``x`` and normalised in one kernel."""
         _dev(x, weight, bias, out, rows)
         D = x.shape[1]
         n = out.shape[0]
@@ -165,6 +185,15 @@ class HipKernels:
             _req(n == x.shape[0], "norm: out must have as many rows as x")
         else:
             _req(rows.dtype == torch.int32 and rows.numel() == n, "norm: rows must be int32, one per output row")
+        if pending is not None:
+            _req(pending.out is x and pending.ldo == D, "norm: the unfinished product belongs to another tensor")
+            rc = self.lib.lev_norm_pending(_ptr(x), _ptr(pending.workspace), pending.n_ranges, _ptr(pending.bias), _ptr(weight), _ptr(bias),
+                                           _ptr(out), _ptr(rows), n, x.shape[0], D, float(eps), int(rms), _DT[out.dtype], _stream())
+            if rc == 0:
+                return
+            if rc < 0:
+                self._check(rc)
+            self.finish(pending)  # no fused kernel at this width: finish the product, then the plain norm
         self._check(self.lib.lev_norm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(rows), n, D, float(eps), int(rms),
                                       _DT[out.dtype], _stream()))
 
@@ -184,8 +213,19 @@ class HipKernels:
         self._ws[device] = new
         return new
 
-    def linear(self, a, w, bias, out, activation: str = "none", residual=None) -> None:
-        """out = act(a @ w.T + bias) (+ residual). a [M, K], w [N, K], out [M, N]; residual float32, may be ``out``."""
+    def finish(self, pending: PendingSum) -> None:
+        """Finish a product that ``linear(..., may_leave_pending=True)`` left unfinished."""
+        x = pending.out
+        self._check(self._unit("gemm_mfma").lev_linear_mfma_finish(_ptr(pending.workspace), _ptr(pending.bias), _ptr(x), pending.ldo, _ptr(x),
+                                                                   pending.ldo, x.shape[0], x.shape[1], pending.n_ranges, 0, _DT[torch.float32],
+                                                                   _stream()))
+
+    def linear(self, a, w, bias, out, activation: str = "none", residual=None, may_leave_pending: bool = False) -> Optional[PendingSum]:
+        """out = act(a @ w.T + bias) (+ residual). a [M, K], w [N, K], out [M, N]; residual float32, may be ``out``.
+
+        ``may_leave_pending`` (only with ``residual is out``, no activation): where the kernel splits the sum over K into
+        ranges, it may stop after writing them and return a ``PendingSum`` instead of running the kernel that adds them
+        up: the caller promises that the next thing to touch ``out`` is ``norm(out, ..., pending=...)`` or ``finish``."""
         # one kernel launch per call: the checks are written to cost little
         if not (a.is_cuda and w.is_cuda and out.is_cuda and (bias is None or bias.is_cuda) and (residual is None or residual.is_cuda)):
             raise KernelError("a kernel was given a tensor that is not on the GPU")
@@ -213,14 +253,14 @@ class HipKernels:
             if self.gemm_library and self.use_library(M, N, K, act):
                 key = (M, N, K, act, bias is None, residual is None, odt)
                 # never while a HIP graph is being recorded: what the library records besides its kernel is not ours to vouch for
-                if key not in self._library_refused and not torch.cuda.is_current_stream_capturing():
+                if key not in self._library_refused and (self.library_in_graphs or not torch.cuda.is_current_stream_capturing()):
                     lib = self._unit("gemm_library")
                     need = lib.lev_linear_library_workspace()
                     ws = self._workspace(need, a.device)
                     rc = lib.lev_linear_library(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws), need,
                                                 M, N, K, act, _DT[odt], _stream())
                     if rc == 0:
-                        return
+                        return None
                     if rc < 0:
                         self._check(rc)
                     self._library_refused.add(key)  # the library has no kernel for it: ours from now on
@@ -229,23 +269,32 @@ class HipKernels:
             if need is None:  # partial sums of a K range split over workgroups
                 need = self._ws_need[(M, N, K)] = gemm.lev_linear_mfma_workspace(M, N, K)
             ws = self._workspace(need, a.device) if need > 0 else None
+            leave = may_leave_pending and need > 0 and residual is out and act == 0 and ldo == N
             self._check(gemm.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
-                                             M, N, K, act, _DT[odt], _stream()))
+                                             M, N, K, act, _DT[odt], int(leave), _stream()))
+            if leave:
+                return PendingSum(out, ws, need // (M * N * 4), bias, ldo)
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
                                                    M, N, K, act, _DT[adt], _DT[odt], _stream()))
+        return None
 
     LIBRARY_ACTIVATIONS = (ACTIVATIONS["none"], ACTIVATIONS["gelu_new"], ACTIVATIONS["relu"])
-    LIBRARY_MIN_ROWS = 256
+    LIBRARY_MIN_ROWS = 25  # up to 24 rows the skinny kernel streams the weights at the rate a plain read reaches
 
     @classmethod
     def use_library(cls, M: int, N: int, K: int, act: int) -> bool:
-        """Which products go to the vendor library: prompt-sized row counts with an epilogue the library has. Measured
-        on MI355X at the widths of GPT-2 7B and XL (see gemm_library.hip): ours are ahead up to a few hundred rows and
-        on narrow outputs of long sums (K >= 4 N) below a thousand rows."""
+        """Which products go to the vendor library: those with an epilogue it has, at the shapes where it was measured
+        ahead on MI355X (widths of GPT-2 7B and XL, with epilogues). From 256 rows: all but long sums into narrow outputs
+        (K >= 4 N) below 1,024 rows and weights of a few MB below 320 rows. From 25 to 255 rows: wide outputs of large
+        weights (N >= 2 K, 32 MB and more: 7B qkv and fc at 64 rows 28.1 / 25.3 and 37.1 / 33.5 us, ours with the kernel that
+        adds its K ranges; at 160 rows 49.7 / 37.2 and 55.7 / 41.6); ours keep N = K (17.4 / 16.3 at 64 rows, 22.1 / 24.6 at
+        128) and K = 4 N (36.8 / 41.2, 43.5 / 81.1)."""
         if act not in cls.LIBRARY_ACTIVATIONS or M < cls.LIBRARY_MIN_ROWS:
             return False
-        if M < 320 and N * K < (1 << 24):  # weights of a few MB: ours up to 320 rows
+        if M < 256:
+            return N >= 2 * K and N * K >= (1 << 24)
+        if M < 320 and N * K < (1 << 24):
             return False
         return not (K >= 4 * N and M < 1024)
 

@@ -74,4 +74,4 @@ class CausalSelfAttention(Mixer):
             if writes_cache:
                 ctx.kernels.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size)
             ctx.kernels.paged_attention(q, a, unit.k_pages, unit.v_pages, ctx.attention, **args)
-        self.out(a, ctx, residual=x)
+        self.out(a, ctx, residual=x, final=True)

@@ -84,9 +84,33 @@ class StepContext:
     nobody: a mixer with state of its own must not count them). With ``attention.positions`` and
     ``attention.token_seq`` this is all a state mixer needs on the device, so that it can be ``graph_safe``."""
     units: Dict[int, CacheUnitView] = field(default_factory=dict)
+    pending: Any = None
+    """A product into the residual stream that its kernel has not finished (``kernels.PendingSum``): the next norm of
+    that tensor folds the rest in, anything else calls ``settle()`` first. Only set while ``may_defer`` is True."""
+    may_defer: bool = False
+    """Set by the decoder around blocks that say ``defers_residual``: the parts of such a block promise that after a
+    product marked ``final`` they do not touch the residual stream again in their ``forward``."""
 
     def empty(self, rows: int, cols: int, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         return torch.empty((rows, cols), dtype=dtype or self.dtype, device=self.device)
+
+    def settle(self) -> None:
+        """Finish what ``pending`` describes, if anything: afterwards the residual stream is up to date."""
+        if self.pending is not None:
+            pending, self.pending = self.pending, None
+            self.kernels.finish(pending)
+
+    def take_pending(self, x: torch.Tensor):
+        """The unfinished product into ``x`` for a norm that folds it in (None if there is none; one into another
+        tensor is settled)."""
+        pending = self.pending
+        if pending is None:
+            return None
+        self.pending = None
+        if pending.out is x:
+            return pending
+        self.kernels.finish(pending)
+        return None
 
 
 class Part:
@@ -104,7 +128,11 @@ class Part:
 
 
 class Norm(Part):
-    """``__call__(x_f32 [T, dim], ctx, rows=None) -> h [T or len(rows), dim]`` in the compute dtype."""
+    """``__call__(x_f32 [T, dim], ctx, rows=None) -> h [T or len(rows), dim]`` in the compute dtype.
+    ``folds_pending``: the norm looks at ``ctx.take_pending(x)`` itself and hands it to its kernel; for one that does
+    not (the default) the block or the decoder calls ``ctx.settle()`` before it runs."""
+
+    folds_pending = False
 
     def __call__(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
@@ -156,6 +184,9 @@ class Block:
 
     kind: str = ""
     roles: tuple = ()
+    defers_residual = False
+    """True: this block only reads the residual stream through norms (after ``ctx.settle()`` unless they fold pending
+    sums in themselves) and through its parts, so a part's last product may leave its sum to the next norm."""
 
     def __init__(self, parts: Dict[str, Part]):
         missing = [r for r in self.roles if r not in parts]

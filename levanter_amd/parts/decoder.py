@@ -75,9 +75,17 @@ class DecoderLm:
         """Run the step's tokens through the plan; float32 logits ``[len(logit_rows), vocab]``."""
         x = self.embedding(ctx)
         for e in self.plan:
-            self.blocks[e.layer].forward(x, ctx, ctx.units[e.cache], e.writes_cache)
+            block = self.blocks[e.layer]
+            ctx.may_defer = bool(block.defers_residual)
+            if not ctx.may_defer:
+                ctx.settle()  # this block may read the residual stream in ways of its own
+            block.forward(x, ctx, ctx.units[e.cache], e.writes_cache)
+        ctx.may_defer = False
         if logit_rows.numel() == 0:
+            ctx.pending = None  # nobody reads the residual stream any more
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=ctx.device)
+        if not self.final_norm.folds_pending:
+            ctx.settle()
         h = self.final_norm(x, ctx, rows=logit_rows)
         return self.head(h, ctx)
 

@@ -31,4 +31,4 @@ class DenseMlp(FeedForward):
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         m = self.up(h, ctx, activation=self.activation)
-        self.down(m, ctx, residual=x)
+        self.down(m, ctx, residual=x, final=True)

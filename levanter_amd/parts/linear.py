@@ -21,8 +21,15 @@ class Linear:
         self.n_out, self.n_in = self.weight.shape
 
     def __call__(self, a: torch.Tensor, ctx: StepContext, *, activation: str = "none", residual: Optional[torch.Tensor] = None,
-                 out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+                 out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None, final: bool = False) -> torch.Tensor:
+        """``final``: the caller does not touch ``residual`` again in its ``forward``. Where the block allows it
+        (``ctx.may_defer``) the product may then leave the sum of its K ranges to the norm that follows."""
+        if ctx.pending is not None:
+            ctx.settle()  # the unfinished product's ranges live in the workspace that this one is about to use
         if out is None:
             out = residual if residual is not None else ctx.empty(a.shape[0], self.n_out, out_dtype)
-        ctx.kernels.linear(a, self.weight, self.bias, out, activation=activation, residual=residual)
+        if final and ctx.may_defer and residual is out:
+            ctx.pending = ctx.kernels.linear(a, self.weight, self.bias, out, activation=activation, residual=residual, may_leave_pending=True)
+        else:
+            ctx.kernels.linear(a, self.weight, self.bias, out, activation=activation, residual=residual)
         return out

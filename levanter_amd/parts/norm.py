@@ -15,6 +15,7 @@ from .spec import PartSpec
 @NORMS.register("layernorm")
 class LayerNorm(Norm):
     graph_safe = True
+    folds_pending = True
 
     rms = False
 
@@ -28,7 +29,11 @@ class LayerNorm(Norm):
     def __call__(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.empty(n, self.dim)
-        ctx.kernels.norm(x, self.weight, self.bias, self.eps, out, rows=rows, rms=self.rms)
+        pending = ctx.take_pending(x)
+        if pending is None:
+            ctx.kernels.norm(x, self.weight, self.bias, self.eps, out, rows=rows, rms=self.rms)
+        else:
+            ctx.kernels.norm(x, self.weight, self.bias, self.eps, out, rows=rows, rms=self.rms, pending=pending)
         return out
 
 

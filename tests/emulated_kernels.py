@@ -69,7 +69,8 @@ class EmulatedKernels:
         out.copy_(x)
 
     # ---- norm
-    def norm(self, x, weight, bias, eps, out, rows=None, rms=False) -> None:
+    def norm(self, x, weight, bias, eps, out, rows=None, rms=False, pending=None) -> None:
+        assert pending is None, "this stand-in never leaves a product unfinished"
         src = x if rows is None else x[rows.long()]
         if rms:
             y = src / torch.sqrt((src * src).mean(-1, keepdim=True) + eps) * weight
@@ -80,7 +81,7 @@ class EmulatedKernels:
         out.copy_(y.to(out.dtype))
 
     # ---- linear
-    def linear(self, a, w, bias, out, activation="none", residual=None) -> None:
+    def linear(self, a, w, bias, out, activation="none", residual=None, may_leave_pending=False) -> None:
         y = a.float() @ w.float().t()
         if bias is not None:
             y = y + bias

@@ -253,9 +253,96 @@ def test_linear_bf16_prompt_sized_rows_with_and_without_the_vendor_library(K, li
         assert n_library == 6 and len(calls) == 6 and all(rc == 0 for rc in calls), calls  # the library took all but the last
 
 
+@pytest.mark.parametrize("M,K_,N,rows", [(64, 4096, 4096, None), (100, 16384, 4096, [99, 3, 3, 50]), (33, 8192, 1608, None),
+                                         (300, 6400, 1600, [299, 0]), (64, 4096, 4104, None), (40, 8192, 8200, None)])
+def test_a_product_that_leaves_its_ranges_to_the_norm(K, M, K_, N, rows):
+    """Where the product into the residual stream splits its sum over K into ranges, it may stop after writing them; the
+    norm that follows adds them to its rows, stores the rows back and normalises them in one kernel. The residual and
+    is bit for bit that of the finished product, the normed rows are those of the plain norm (up to the order in which the
+    statistics are summed), for all rows and for a selection, also at a width where the norm falls back to finishing the product first (more than 8,192 columns)."""
+    a = _rand(M, K_, dtype=torch.bfloat16, seed=M).to(DEV)
+    w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=N).to(DEV)
+    bias = _rand(N, seed=3).to(DEV)
+    gamma, beta = (1 + 0.1 * _rand(N, seed=5)).to(DEV), _rand(N, seed=6).to(DEV)
+    x0 = _rand(M, N, seed=4).to(DEV)
+    ridx = None if rows is None else torch.tensor(rows, dtype=torch.int32, device=DEV)
+    n_out = M if rows is None else len(rows)
+    # the finished product, then the norm
+    x_ref = x0.clone()
+    assert K.linear(a, w, bias, x_ref, residual=x_ref) is None
+    h_ref = torch.empty(n_out, N, dtype=torch.bfloat16, device=DEV)
+    K.norm(x_ref, gamma, beta, 1e-5, h_ref, rows=ridx)
+    # the same with the sum left to the norm
+    x = x0.clone()
+    pending = K.linear(a, w, bias, x, residual=x, may_leave_pending=True)
+    assert pending is not None and pending.n_ranges > 1, "this shape was meant to split K"
+    assert torch.equal(x, x0)  # nothing has been added yet
+    h = torch.empty(n_out, N, dtype=torch.bfloat16, device=DEV)
+    K.norm(x, gamma, beta, 1e-5, h, rows=ridx, pending=pending)
+    # the fused kernel sums the row's statistics over 1,024 threads, the plain one over 256: one bfloat16 step at most
+    assert float((h.float() - h_ref.float()).abs().max()) <= 2.0 ** -7 * float(h_ref.float().abs().max())
+    assert float((h != h_ref).float().mean()) < 1e-3
+    touched = slice(None) if rows is None or N > 8192 else torch.tensor(sorted(set(rows)), device=DEV)
+    assert torch.equal(x[touched], x_ref[touched])
+    want = x0.double() + a.double() @ w.double().t() + bias.double()
+    assert float((x[touched].double() - want[touched]).abs().max() / want.abs().max()) < 2e-3
+    # finishing it by itself gives the same residual
+    x2 = x0.clone()
+    K.finish(K.linear(a, w, bias, x2, residual=x2, may_leave_pending=True))
+    assert torch.equal(x2, x_ref)
+    # a product that does not split K, or has an activation, or another output, is finished as always
+    assert K.linear(a[:8], w, bias, x2[:8], residual=x2[:8], may_leave_pending=True) is None
+    out = torch.empty(M, N, device=DEV)
+    assert K.linear(a, w, bias, out, residual=x0, may_leave_pending=True) is None
+
+
+@pytest.mark.parametrize("M,K_,N,act,res", [(64, 4096, 12288, "none", False), (160, 4096, 16384, "gelu_new", False),
+                                            (300, 1600, 6400, "none", True), (128, 4096, 4096, "none", True)])
+def test_the_vendor_library_s_product_inside_a_recorded_graph(K, M, K_, N, act, res, monkeypatch):
+    """A recorded graph replays only kernels and copies faithfully; what else a library call records (clearing of
+    flags or partial sums by memset nodes) has gone wrong on later replays on this hardware. The library's product
+    is therefore recorded and replayed six times, with changed inputs, eager products of other shapes and
+    synchronisations between the replays; every replay must give the eager result bit for bit."""
+    monkeypatch.setattr(K, "use_library", lambda M, N, K_, act: True)
+    assert K.library_in_graphs
+    a = _rand(M, K_, dtype=torch.bfloat16, seed=1).to(DEV)
+    w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=2).to(DEV)
+    bias = _rand(N, seed=3).to(DEV)
+    x0 = _rand(M, N, seed=4).to(DEV)
+    out = torch.zeros(M, N, device=DEV, dtype=torch.float32 if res else torch.bfloat16)
+    other_a = _rand(512, 1024, dtype=torch.bfloat16, seed=5).to(DEV)
+    other_w = _rand(768, 1024, dtype=torch.bfloat16, seed=6).to(DEV)
+    other_out = torch.zeros(512, 768, device=DEV, dtype=torch.bfloat16)
+
+    def product():
+        if res:
+            out.copy_(x0)
+            K.linear(a, w, bias, out, residual=out)
+        else:
+            K.linear(a, w, bias, out, activation=act)
+
+    product()  # eager first: kernels and the library's plan are loaded
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        product()
+    for i in range(6):
+        a.copy_(_rand(M, K_, dtype=torch.bfloat16, seed=10 + i).to(DEV))
+        product()
+        want = out.clone()
+        out.zero_()
+        K.linear(other_a, other_w, None, other_out)  # eager work of the program's own between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
+        assert bool(out.float().abs().sum() > 0)
+
+
 def test_which_products_go_to_the_vendor_library(K):
     none, gelu, silu = 0, 1, 4
-    assert not K.use_library(255, 12288, 4096, none) and K.use_library(256, 12288, 4096, none)
+    assert not K.use_library(24, 12288, 4096, none) and K.use_library(25, 12288, 4096, none) and K.use_library(256, 12288, 4096, none)
+    assert not K.use_library(64, 4096, 4096, none) and not K.use_library(64, 4096, 16384, none) and not K.use_library(64, 4800, 1600, none)
     assert K.use_library(2048, 16384, 4096, gelu) and not K.use_library(2048, 16384, 4096, silu)
     assert not K.use_library(512, 4096, 16384, none) and K.use_library(1024, 4096, 16384, none)  # long sums into a narrow output
     assert not K.use_library(256, 4800, 1600, none) and K.use_library(320, 4800, 1600, none)  # small weights
