@@ -211,11 +211,13 @@ def serving_workload(args) -> int:
         return [Request(prompt_tokens=torch.randint(0, V, (n,), generator=g).tolist(), request_id=i, max_new_tokens=new_tokens,
                         temperature=temperature) for i, n in enumerate(lens)]
 
-    # a short run first: kernels are loaded and the decode shapes have been seen once
-    warm = [Request(prompt_tokens=r.prompt_tokens[:32], request_id=r.request_id, max_new_tokens=4, temperature=temperature)
-            for r in requests(1)[:4]]
+    # a short run first: kernels and the GEMM library are loaded (prompt portions of the workload's size among them) and
+    # the decode shapes have been seen once
+    warm = [Request(prompt_tokens=r.prompt_tokens[:chunk if i < 2 else 32], request_id=r.request_id, max_new_tokens=4, temperature=temperature)
+            for i, r in enumerate(requests(1)[:4])]
     engine.generate(warm)
     engine.reset()
+    engine.warm_up()
     step_ms = []
     seqs = engine.enqueue_requests(requests(2))
     torch.cuda.synchronize()

@@ -183,6 +183,27 @@ class InferenceEngine:
                                 logprobs=[list(s.logprobs) for s in seqs] if want_lp else None,
                                 total_generated=total, finish_reasons=[s.finish_reason for s in seqs])
 
+    def warm_up(self, token_counts: Optional[Sequence[int]] = None) -> None:
+        """Run prompts of several lengths once and drop them: kernels, and the GEMM library's code for the row counts
+        that prompt portions will have, are loaded before the first request is timed (a first use can take a fifth of a
+        second). ``token_counts``: tokens of each warm-up step; default: a ladder from 32 up to the largest portion."""
+        limit = min(self.config.imputed_max_prefill_size, self.runner.max_len - 1)
+        if token_counts is None:
+            token_counts = [n for n in (32, 64, 128, 192, 256, 288, 320, 384, 448, 512, 640, 768, 1024, 1280, 1536, 2048) if n <= limit]
+            if limit not in token_counts:
+                token_counts.append(limit)
+        if not self.scheduler.idle or self._pending is not None:
+            raise RuntimeError("warm_up() runs on an idle engine")
+        v = self.model.vocab_size
+        for n in token_counts:
+            n = max(1, min(int(n), limit))
+            self.generate([Request(prompt_tokens=[(7 * i + 3) % v for i in range(n)], request_id=-1, max_new_tokens=1)])
+        # batches of decoding requests: the head and the products of a decode step at the row counts where the library takes them
+        most = self.config.max_seqs
+        for b in sorted({b for b in (most, most // 2, 48, 32, 25) if 25 <= b <= most}):
+            self.generate([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=3) for i in range(b)])
+        self.reset()
+
     def reset(self) -> None:
         """Drop every request and give back all pages and slots (engine.py:761-776)."""
         if self._pending is not None and self._pending.sample is not None:

@@ -151,6 +151,24 @@ def test_greedy_generation_through_the_entry_point(dtype):
     assert engine.cache.n_free_slots == 4
 
 
+def test_warm_up_leaves_the_engine_as_it_found_it():
+    from levanter_amd.engine import Request
+
+    d = write_model(TINY_A, 0, torch.float32)
+    reqs = [Request(prompt_tokens=[5, 6, 7, 8], request_id=0, max_new_tokens=8, temperature=0.9, key=3)]
+    cold = _engine(d, "float32", max_seqs=32).generate(reqs).tokens
+    engine = _engine(d, "float32", max_seqs=32)
+    engine.warm_up()
+    assert engine.scheduler.idle and engine.cache.n_free_slots == 32
+    engine.cache.check_invariants()
+    assert all(int(g.pool.ref_counts.sum()) == 0 for g in engine.cache.groups)
+    assert engine.generate(reqs).tokens == cold
+    engine.enqueue_requests(reqs)
+    engine.step()
+    with pytest.raises(RuntimeError, match="idle"):
+        engine.warm_up()
+
+
 def _random_requests(rng, vocab, max_pos, n):
     from levanter_amd.engine import SeqDecodingParams
 
