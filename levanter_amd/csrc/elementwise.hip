@@ -487,6 +487,20 @@ extern "C" int lev_sample(const float* logits, long row_stride, const float* tem
   return lev_check_launch("sample merge");
 }
 
+// ------------------------------------------------------------------------------------------
+// Token ids of a step that were sampled by the step before and are still on the device: dst[i] = src[rows ? rows[i] : i].
+__global__ void feed_tokens_kernel(int* __restrict__ dst, const int* __restrict__ src, const int* __restrict__ rows, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[rows ? rows[i] : i];
+}
+
+extern "C" int lev_feed_tokens(int* dst, const int* src, const int* rows, int n, hipStream_t stream) {
+  LEV_REQUIRE(n >= 0 && (n == 0 || (dst && src)), "feed_tokens: bad arguments (n=%d)", n);
+  if (n == 0) return 0;
+  feed_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, src, rows, n);
+  return lev_check_launch("feed_tokens");
+}
+
 // ---- the same sampling from a scratch array of the library's own (see sample_static.h) -----------------------
 // In host code `sample_scratch` is only a stand-in for the symbol: the address a kernel can use comes from
 // hipGetSymbolAddress, once per device, and is kept in g_sample_scratch[device].

@@ -149,7 +149,7 @@ class InferenceEngine:
         if feed is not None:
             device_tokens, rows = feed
             same = rows == list(range(len(rows))) and len(rows) == int(device_tokens.numel())
-            token_feed = (device_tokens, None if same else torch.tensor(rows, dtype=torch.int64, device=device_tokens.device), len(rows))
+            token_feed = (device_tokens, None if same else torch.tensor(rows, dtype=torch.int32, device=device_tokens.device), len(rows))
         logits = self.runner.step(entries, copy_out=False, token_feed=token_feed)
         wanted = [e for e in plan if e.wants_logits]
         sample = None

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from levanter_amd.cache import NO_PAGE, CacheManager, OutOfPages, SequenceHandle
+from levanter_amd.kernels.staging import pinned_pool
 from levanter_amd.parts.base import AttentionMeta, BuildEnv, CacheUnitView, GroupView, StepContext
 from levanter_amd.parts.decoder import DecoderLm
 
@@ -232,23 +233,17 @@ class ModelRunner:
         return ctx
 
     def _upload(self, host: np.ndarray) -> torch.Tensor:
-        t = torch.from_numpy(host)
         if self.env.device.type == "cpu":
-            return t
-        return t.pin_memory().to(self.env.device, non_blocking=True)
+            return torch.from_numpy(host)
+        return pinned_pool().upload(host, self.env.device)
 
     # ---- decode steps as HIP graphs --------------------------------------------------------
-    @staticmethod
-    def _feed_tokens(dev: torch.Tensor, b: "HostBatch", token_feed) -> None:
+    def _feed_tokens(self, dev: torch.Tensor, b: "HostBatch", token_feed) -> None:
         """Entry i's token id (i < n) comes from ``device_tokens[rows[i]]``: these entries are the step's first tokens."""
         if token_feed is None:
             return
         device_tokens, rows, n = token_feed
-        dst = dev[b.offs[0]:b.offs[0] + n]
-        if rows is None:  # the same requests in the same order as in the step before
-            dst.copy_(device_tokens[:n])
-        else:
-            torch.index_select(device_tokens, 0, rows, out=dst)
+        self.env.kernels.feed_tokens(dev[b.offs[0]:b.offs[0] + n], device_tokens, rows, n)
 
     def _run_graphed(self, b: "HostBatch", token_feed=None) -> torch.Tensor:
         """A step of single tokens has a kernel sequence that depends only on (requests, wanted rows,

@@ -91,6 +91,7 @@ class HipKernels:
             "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
             "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
             "lev_sample_workspace": [c_int],
+            "lev_feed_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_void_p],
             "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
             "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
             + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
@@ -100,6 +101,7 @@ class HipKernels:
         # the vendor library's GEMM for prompt-sized row counts (see use_library); "0" keeps every product on our kernels
         self.gemm_library = os.environ.get("LEVANTER_AMD_GEMM_LIBRARY", "1") != "0"
         self._library_refused = set()
+        self._slow_attention_warned = set()
         # The library's product may be recorded into HIP graphs: replays with changed inputs and eager work between them
         # give the eager results bit for bit (tests/test_gpu_kernels.py records and replays it at four shapes).
         self.library_in_graphs = True
@@ -168,6 +170,14 @@ class HipKernels:
             _req(pos_table.is_contiguous() and pos_table.shape[1] == D and pos_table.dtype == table.dtype, "embed: bad position table")
         self._check(self.lib.lev_embed(_ptr(tokens), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(out), T, D,
                                        _DT[table.dtype], _stream()))
+
+    def feed_tokens(self, dst, src, rows, n: int) -> None:
+        """dst[i] = src[rows[i]] (``rows`` None: src[i]) for i < n: int32 token ids that never leave the device."""
+        _dev(dst, src, rows)
+        _req(dst.dtype == src.dtype == torch.int32 and dst.numel() >= n and dst.is_contiguous() and src.is_contiguous(), "feed_tokens: int32 vectors")
+        _req(rows is None or (rows.dtype == torch.int32 and rows.numel() >= n), "feed_tokens: rows must be int32, one per token")
+        _req(rows is not None or src.numel() >= n, "feed_tokens: too few source tokens")
+        self._check(self.lib.lev_feed_tokens(_ptr(dst), _ptr(src), _ptr(rows), int(n), _stream()))
 
     # ---- norms ---------------------------------------------------------------------------
     def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False, pending: Optional[PendingSum] = None) -> None:
@@ -333,6 +343,8 @@ class HipKernels:
         qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
         mfma = (q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
                 and page_size & (page_size - 1) == 0)  # the matrix-core kernels index pages with shifts
+        if q.dtype == torch.bfloat16 and self.use_mfma and not mfma:
+            self._warn_slow_attention(head_dim, n_heads // n_kv_heads, page_size)
         if k_new is not None:
             fusable = mfma and meta.n_prefill_tiles == 0 and meta.n_decode == T
             if not fusable:
@@ -374,6 +386,16 @@ class HipKernels:
             # batch 1, 1,850 keys: 3.73 -> 3.26 ms a step; batch 4, 580 keys: 3.39 ms with the clamp, 3.43 without).
             splits = 8
         return splits
+
+    def _warn_slow_attention(self, head_dim: int, group: int, page_size: int) -> None:
+        key = (head_dim, group, page_size)
+        if key not in self._slow_attention_warned:
+            self._slow_attention_warned.add(key)
+            import warnings
+
+            warnings.warn(f"attention with head_dim={head_dim}, {group} query heads per kv head and page_size={page_size} has no matrix-core "
+                          f"kernel (head sizes 16..128 in steps of 16, at most 16 query heads per kv head, page sizes that are powers of "
+                          f"two): it runs on the plain-arithmetic kernel, which is correct and slow", RuntimeWarning, stacklevel=3)
 
     @staticmethod
     def mfma_attention_supports(head_dim: int, group: int) -> bool:

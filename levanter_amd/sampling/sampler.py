@@ -15,6 +15,8 @@ from typing import Sequence, Tuple
 import numpy as np
 import torch
 
+from levanter_amd.kernels.staging import pinned_pool
+
 _MASK64 = (1 << 64) - 1
 
 
@@ -57,8 +59,7 @@ class Sampler:
         host[:r] = np.asarray(temperatures, np.float32).view(np.int32)
         host[r:3 * r] = np.asarray([[_as_i32(k[0]), _as_i32(k[1])] for k in keys], np.int64).reshape(-1)
         host[3 * r:] = np.asarray(positions, np.int64)
-        t = torch.from_numpy(host)
-        dev = t if self.device.type == "cpu" else t.pin_memory().to(self.device, non_blocking=True)
+        dev = torch.from_numpy(host) if self.device.type == "cpu" else pinned_pool().upload(host, self.device)
         out = torch.empty(2 * r, dtype=torch.int32, device=self.device)  # tokens, then log-probabilities: one copy back
         tokens, logprobs = out[:r], out[r:].view(torch.float32)
         self.kernels.sample(logits, dev[:r].view(torch.float32), dev[r:3 * r].view(r, 2), dev[3 * r:], tokens, logprobs)
@@ -77,8 +78,8 @@ class Sampler:
         out = self._last_out
         if self.device.type == "cpu":
             return PendingSample(r, tokens, out.clone(), None)
-        host = torch.empty(2 * r, dtype=torch.int32).pin_memory()
-        host.copy_(out, non_blocking=True)
+        host = pinned_pool().acquire(2 * r)
+        host[:2 * r].copy_(out, non_blocking=True)
         done = torch.cuda.Event()
         done.record()
         return PendingSample(r, tokens, host, done)
@@ -88,7 +89,11 @@ class Sampler:
         if pending.done is not None:
             pending.done.synchronize()
         r = pending.rows
-        return pending.host[:r].tolist(), pending.host[r:].view(torch.float32).tolist()
+        result = pending.host[:r].tolist(), pending.host[r:2 * r].view(torch.float32).tolist()
+        if pending.done is not None and pending.host is not None:
+            pinned_pool().release(pending.host)  # a pinned buffer of the pool: the next sampling may take it
+            pending.host = None
+        return result
 
 
 class PendingSample:

@@ -68,6 +68,9 @@ class EmulatedKernels:
             x = x + pos_table[positions.long()].float()
         out.copy_(x)
 
+    def feed_tokens(self, dst, src, rows, n) -> None:
+        dst[:n] = src[:n] if rows is None else src[rows[:n].long()]
+
     # ---- norm
     def norm(self, x, weight, bias, eps, out, rows=None, rms=False, pending=None) -> None:
         assert pending is None, "this stand-in never leaves a product unfinished"
