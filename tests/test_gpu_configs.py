@@ -208,7 +208,7 @@ def test_command_line_from_a_yaml_file_with_overrides_in_bfloat16(tmp_path):
         toks, reason = rounds[0][i]
         assert reason == "length" and len(toks) == 20  # the command line's value, not the file's
         clear += _check_greedy(w, TINY_A, p, toks, P.bf16_rounding, margin=2e-2)
-    assert clear >= 10
+    assert clear >= 45, clear  # of 60
     # a stop sequence: the 4th and 5th generated token of sequence 0 end it where they first appear one after the other
     first = rounds[0][0][0]
     stop = first[3:5]

@@ -145,8 +145,9 @@ def test_greedy_generation_through_the_entry_point(dtype):
         for p, out in zip(prompts, res.tokens):
             assert out == P.plain_greedy_generate(w, TINY_A, p, 16)
     else:
+        # 47 of the 48 tokens have a margin that clear along the plain implementation's own path
         clear = sum(_check_greedy(w, TINY_A, p, out, P.bf16_rounding, margin=2e-2) for p, out in zip(prompts, res.tokens))
-        assert clear >= 10
+        assert clear >= 40
     engine.cache.check_invariants()
     assert engine.cache.n_free_slots == 4
 
