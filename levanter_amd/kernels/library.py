@@ -41,18 +41,19 @@ class PendingSum:
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else c_void_p(t.data_ptr())
+    """A tensor's address as ctypes takes it for a ``c_void_p`` parameter: a plain integer, or None."""
+    return None if t is None else t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream():
-    """The current HIP stream as a pointer. ``torch.cuda.current_stream()`` builds a Stream object on every call
+    """The current HIP stream as an integer. ``torch.cuda.current_stream()`` builds a Stream object on every call
     (several microseconds, once per kernel launch); the raw getter is a plain C call."""
     if _raw_stream is not None:
-        return c_void_p(_raw_stream(torch.cuda.current_device()))
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(torch.cuda.current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _req(cond: bool, msg: str) -> None:
@@ -68,9 +69,13 @@ def _dev(*ts) -> None:
 
 def _rows(t: torch.Tensor, name: str) -> int:
     """Row stride (in elements) of a 2-D tensor whose rows are contiguous."""
-    _req(t.dim() == 2, f"{name} must have 2 dimensions, has {t.dim()}")
-    _req(t.shape[1] == 1 or t.stride(1) == 1, f"{name}: rows must be contiguous")
-    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    st = t.stride()
+    if len(st) != 2:
+        raise KernelError(f"{name} must have 2 dimensions, has {len(st)}")
+    n_rows, n_cols = t.shape
+    if st[1] != 1 and n_cols != 1:
+        raise KernelError(f"{name}: rows must be contiguous")
+    return st[0] if n_rows > 1 else max(st[0], n_cols)
 
 
 class HipKernels:
@@ -107,7 +112,10 @@ class HipKernels:
         self.library_in_graphs = True
         self._sample_ws = None
         self._units = {}
+        self._held_stream = None  # see hold_stream
+        self._library_ws_bytes = None
         self._ws, self._ws_outgrown, self._ws_need = {}, [], {}  # GEMM scratch memory per device, see _workspace
+        self._ws_last = None
         L.lev_attention_prefill_tile_rows.restype = c_int
         self.prefill_tile_rows = int(L.lev_attention_prefill_tile_rows())
 
@@ -150,6 +158,18 @@ class HipKernels:
             self._units[unit] = lib
         return lib
 
+    def hold_stream(self) -> None:
+        """Look the current stream up once and use it for every launch until ``release_stream``: a model's forward pass
+        launches hundreds of kernels on one stream, and the lookup is a tenth of a launch's cost on the host."""
+        self._held_stream = _stream()
+
+    def release_stream(self) -> None:
+        self._held_stream = None
+
+    def _s(self):
+        held = self._held_stream
+        return _stream() if held is None else held
+
     def loaded_units(self):
         return ["core", *self._units]
 
@@ -169,7 +189,7 @@ class HipKernels:
         if pos_table is not None:
             _req(pos_table.is_contiguous() and pos_table.shape[1] == D and pos_table.dtype == table.dtype, "embed: bad position table")
         self._check(self.lib.lev_embed(_ptr(tokens), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(out), T, D,
-                                       _DT[table.dtype], _stream()))
+                                       _DT[table.dtype], self._s()))
 
     def feed_tokens(self, dst, src, rows, n: int) -> None:
         """dst[i] = src[rows[i]] (``rows`` None: src[i]) for i < n: int32 token ids that never leave the device."""
@@ -177,7 +197,7 @@ class HipKernels:
         _req(dst.dtype == src.dtype == torch.int32 and dst.numel() >= n and dst.is_contiguous() and src.is_contiguous(), "feed_tokens: int32 vectors")
         _req(rows is None or (rows.dtype == torch.int32 and rows.numel() >= n), "feed_tokens: rows must be int32, one per token")
         _req(rows is not None or src.numel() >= n, "feed_tokens: too few source tokens")
-        self._check(self.lib.lev_feed_tokens(_ptr(dst), _ptr(src), _ptr(rows), int(n), _stream()))
+        self._check(self.lib.lev_feed_tokens(_ptr(dst), _ptr(src), _ptr(rows), int(n), self._s()))
 
     # ---- norms ---------------------------------------------------------------------------
     def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False, pending: Optional[PendingSum] = None) -> None:
@@ -198,22 +218,26 @@ class HipKernels:
         if pending is not None:
             _req(pending.out is x and pending.ldo == D, "norm: the unfinished product belongs to another tensor")
             rc = self.lib.lev_norm_pending(_ptr(x), _ptr(pending.workspace), pending.n_ranges, _ptr(pending.bias), _ptr(weight), _ptr(bias),
-                                           _ptr(out), _ptr(rows), n, x.shape[0], D, float(eps), int(rms), _DT[out.dtype], _stream())
+                                           _ptr(out), _ptr(rows), n, x.shape[0], D, float(eps), int(rms), _DT[out.dtype], self._s())
             if rc == 0:
                 return
             if rc < 0:
                 self._check(rc)
             self.finish(pending)  # no fused kernel at this width: finish the product, then the plain norm
         self._check(self.lib.lev_norm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(rows), n, D, float(eps), int(rms),
-                                      _DT[out.dtype], _stream()))
+                                      _DT[out.dtype], self._s()))
 
     # ---- linear ----------------------------------------------------------------------------
     def _workspace(self, need: int, device) -> torch.Tensor:
         """Scratch memory for partial sums: one buffer per device that only grows. Kernels on one stream take turns
         with it. A buffer that is outgrown stays alive, because recorded HIP graphs may point at it; while a graph is
         being recorded a buffer that is too small is not replaced but a fresh one handed out, which stays with the graph."""
+        last = self._ws_last
+        if last is not None and last[0] is device and last[2] >= need:
+            return last[1]
         ws = self._ws.get(device)
         if ws is not None and ws.numel() >= need:
+            self._ws_last = (device, ws, ws.numel())
             return ws
         if torch.cuda.is_current_stream_capturing():
             return torch.empty(need, dtype=torch.uint8, device=device)
@@ -221,6 +245,7 @@ class HipKernels:
             self._ws_outgrown.append(ws)
         new = torch.empty(max(need, 2 * (ws.numel() if ws is not None else 0)), dtype=torch.uint8, device=device)
         self._ws[device] = new
+        self._ws_last = None
         return new
 
     def finish(self, pending: PendingSum) -> None:
@@ -228,7 +253,7 @@ class HipKernels:
         x = pending.out
         self._check(self._unit("gemm_mfma").lev_linear_mfma_finish(_ptr(pending.workspace), _ptr(pending.bias), _ptr(x), pending.ldo, _ptr(x),
                                                                    pending.ldo, x.shape[0], x.shape[1], pending.n_ranges, 0, _DT[torch.float32],
-                                                                   _stream()))
+                                                                   self._s()))
 
     def linear(self, a, w, bias, out, activation: str = "none", residual=None, may_leave_pending: bool = False) -> Optional[PendingSum]:
         """out = act(a @ w.T + bias) (+ residual). a [M, K], w [N, K], out [M, N]; residual float32, may be ``out``.
@@ -264,29 +289,31 @@ class HipKernels:
                 key = (M, N, K, act, bias is None, residual is None, odt)
                 # never while a HIP graph is being recorded: what the library records besides its kernel is not ours to vouch for
                 if key not in self._library_refused and (self.library_in_graphs or not torch.cuda.is_current_stream_capturing()):
-                    lib = self._unit("gemm_library")
-                    need = lib.lev_linear_library_workspace()
+                    lib = self._units.get("gemm_library") or self._unit("gemm_library")
+                    need = self._library_ws_bytes
+                    if need is None:
+                        need = self._library_ws_bytes = lib.lev_linear_library_workspace()
                     ws = self._workspace(need, a.device)
                     rc = lib.lev_linear_library(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws), need,
-                                                M, N, K, act, _DT[odt], _stream())
+                                                M, N, K, act, _DT[odt], self._s())
                     if rc == 0:
                         return None
                     if rc < 0:
                         self._check(rc)
                     self._library_refused.add(key)  # the library has no kernel for it: ours from now on
-            gemm = self._unit("gemm_mfma")
+            gemm = self._units.get("gemm_mfma") or self._unit("gemm_mfma")
             need = self._ws_need.get((M, N, K))
             if need is None:  # partial sums of a K range split over workgroups
                 need = self._ws_need[(M, N, K)] = gemm.lev_linear_mfma_workspace(M, N, K)
             ws = self._workspace(need, a.device) if need > 0 else None
             leave = may_leave_pending and need > 0 and residual is out and act == 0 and ldo == N
             self._check(gemm.lev_linear_mfma(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo, _ptr(ws),
-                                             M, N, K, act, _DT[odt], int(leave), _stream()))
+                                             M, N, K, act, _DT[odt], int(leave), self._s()))
             if leave:
                 return PendingSum(out, ws, need // (M * N * 4), bias, ldo)
         else:
             self._check(self.lib.lev_linear_simple(_ptr(a), lda, _ptr(w), _ptr(bias), _ptr(residual), ldr, _ptr(out), ldo,
-                                                   M, N, K, act, _DT[adt], _DT[odt], _stream()))
+                                                   M, N, K, act, _DT[adt], _DT[odt], self._s()))
         return None
 
     LIBRARY_ACTIVATIONS = (ACTIVATIONS["none"], ACTIVATIONS["gelu_new"], ACTIVATIONS["relu"])
@@ -311,16 +338,21 @@ class HipKernels:
     # ---- cache write -----------------------------------------------------------------------
     def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int) -> None:
         """Scatter the new tokens' keys and values ([T, n_kv_heads*head_dim] views) to ``dest[t] = page*page_size + offset``."""
-        _dev(k, v, k_pages, v_pages, dest)
-        T = k.shape[0]
-        _req(k.shape == v.shape and k.shape[1] == n_kv_heads * head_dim, "kv_write: k and v must be [T, kv_heads*head_dim]")
-        _req(k.dtype == v.dtype == k_pages.dtype == v_pages.dtype and k.dtype in _DT, "kv_write: dtypes differ")
-        _req(dest.dtype == torch.int32 and dest.numel() == T, "kv_write: one int32 destination per token")
-        _req(k_pages.is_contiguous() and v_pages.is_contiguous(), "kv_write: pages must be contiguous")
-        per_page = n_kv_heads * head_dim * page_size
-        _req(k_pages.numel() % per_page == 0 and k_pages.numel() == v_pages.numel(), "kv_write: page tensors do not fit the sizes")
+        if not (k.is_cuda and v.is_cuda and k_pages.is_cuda and v_pages.is_cuda and dest.is_cuda):
+            raise KernelError("a kernel was given a tensor that is not on the GPU")
+        T, cols = k.shape
+        dt = k.dtype
+        if not (v.shape == k.shape and cols == n_kv_heads * head_dim):
+            raise KernelError("kv_write: k and v must be [T, kv_heads*head_dim]")
+        if not (dt == v.dtype == k_pages.dtype == v_pages.dtype and dt in _DT):
+            raise KernelError("kv_write: dtypes differ")
+        if not (dest.dtype == torch.int32 and dest.numel() == T):
+            raise KernelError("kv_write: one int32 destination per token")
+        n_elems = k_pages.numel()
+        if not (k_pages.is_contiguous() and v_pages.is_contiguous() and n_elems % (cols * page_size) == 0 and n_elems == v_pages.numel()):
+            raise KernelError("kv_write: page tensors must be contiguous and fit the sizes")
         self._check(self.lib.lev_kv_write(_ptr(k), _ptr(v), _rows(k, "kv_write: k"), _rows(v, "kv_write: v"), _ptr(k_pages),
-                                          _ptr(v_pages), _ptr(dest), T, n_kv_heads, head_dim, page_size, _DT[k.dtype], _stream()))
+                                          _ptr(v_pages), _ptr(dest), T, n_kv_heads, head_dim, page_size, _DT[dt], self._s()))
 
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,
@@ -332,43 +364,59 @@ class HipKernels:
         ``k_new``/``v_new``/``dest``: the step's new keys and values, not yet written. Returns True if this
         call has written them to their pages (a step of single tokens on the matrix-core path does it inside
         the attention kernel); False means the caller must call ``kv_write`` first and call again without them."""
-        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, k_new, v_new, dest)
-        T = q.shape[0]
-        _req(q.shape[1] == n_heads * head_dim and out.shape == q.shape, "attention: q and out must be [T, heads*head_dim]")
-        _req(q.dtype == out.dtype == k_pages.dtype == v_pages.dtype and q.dtype in _DT, "attention: dtypes differ")
-        _req(meta.positions.numel() == T and meta.token_seq.numel() == T, "attention: one position and request row per token")
-        _req(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "attention: bad block tables")
-        _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
+        if not (q.is_cuda and out.is_cuda and k_pages.is_cuda and v_pages.is_cuda):
+            raise KernelError("a kernel was given a tensor that is not on the GPU")
+        T, cols = q.shape
+        dt = q.dtype
+        if not (cols == n_heads * head_dim and out.shape == q.shape):
+            raise KernelError("attention: q and out must be [T, heads*head_dim]")
+        if not (dt == out.dtype == k_pages.dtype == v_pages.dtype and dt in _DT):
+            raise KernelError("attention: dtypes differ")
+        # what depends on the step and the cache group only (tables, work lists, the split of the key range, scratch memory) is
+        # checked and decided at the step's first layer and kept with the step's description
+        key = (n_heads, n_kv_heads, head_dim, page_size, id(block_tables), dt)
+        plan = meta.plans.get(key)
+        if plan is None:
+            _dev(block_tables, meta.positions, meta.token_seq)
+            _req(meta.positions.numel() == T and meta.token_seq.numel() == T, "attention: one position and request row per token")
+            _req(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "attention: bad block tables")
+            _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
+            mfma = (dt == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
+                    and page_size & (page_size - 1) == 0)  # the matrix-core kernels index pages with shifts
+            if dt == torch.bfloat16 and self.use_mfma and not mfma:
+                self._warn_slow_attention(head_dim, n_heads // n_kv_heads, page_size)
+            splits, ws, lib = 1, None, None
+            if mfma:
+                splits = self.decode_splits(meta, n_heads, n_kv_heads)
+                need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
+                ws = meta.workspace(need, q.device)
+                lib = self._unit(_build.attention_unit(head_dim))
+            plan = meta.plans[key] = (mfma, splits, ws, _ptr(ws), lib, _ptr(block_tables), block_tables.shape[1], _ptr(meta.positions),
+                                      _ptr(meta.token_seq), _ptr(meta.prefill_tiles), _ptr(meta.decode_tokens), block_tables)
+        mfma, splits, _ws, ws_ptr, lib, bt_ptr, bt_width, pos_ptr, seq_ptr, tiles_ptr, decode_ptr, _bt = plan
         w = int(window) if window else 0
         qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
-        mfma = (q.dtype == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
-                and page_size & (page_size - 1) == 0)  # the matrix-core kernels index pages with shifts
-        if q.dtype == torch.bfloat16 and self.use_mfma and not mfma:
-            self._warn_slow_attention(head_dim, n_heads // n_kv_heads, page_size)
+        kvs = 0
         if k_new is not None:
             fusable = mfma and meta.n_prefill_tiles == 0 and meta.n_decode == T
             if not fusable:
                 return False
-            _req(k_new.shape == v_new.shape == (T, n_kv_heads * head_dim) and k_new.dtype == v_new.dtype == q.dtype,
+            _dev(k_new, v_new, dest)
+            _req(k_new.shape == v_new.shape == (T, n_kv_heads * head_dim) and k_new.dtype == v_new.dtype == dt,
                  "attention: new keys and values must be [T, kv_heads*head_dim] of the compute dtype")
             _req(dest is not None and dest.dtype == torch.int32 and dest.numel() == T, "attention: one int32 destination per token")
             kvs = _rows(k_new, "attention: k_new")
             _req(kvs == _rows(v_new, "attention: v_new"), "attention: new keys and values must share a row stride")
         if mfma:
-            splits = self.decode_splits(meta, n_heads, n_kv_heads)
-            need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
-            ws = meta.workspace(need, q.device)
-            self._check(self._unit(_build.attention_unit(head_dim)).lev_attention_mfma(
-                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
-                _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles,
-                _ptr(meta.decode_tokens), meta.n_decode, _ptr(k_new), _ptr(v_new), kvs if k_new is not None else 0,
-                _ptr(dest) if k_new is not None else None, _ptr(ws), n_heads, n_kv_heads, head_dim, page_size,
-                splits, float(scale), w, _stream()))
+            self._check(lib.lev_attention_mfma(
+                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, tiles_ptr,
+                meta.n_prefill_tiles, decode_ptr, meta.n_decode, _ptr(k_new), _ptr(v_new), kvs,
+                _ptr(dest) if k_new is not None else None, ws_ptr, n_heads, n_kv_heads, head_dim, page_size,
+                splits, float(scale), w, self._s()))
             return k_new is not None
         self._check(self.lib.lev_attention_simple(
-            _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
-            _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, page_size, float(scale), w,
-            _DT[q.dtype], _stream()))
+            _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, T, n_heads, n_kv_heads,
+            head_dim, page_size, float(scale), w, _DT[dt], self._s()))
         return False
 
     @staticmethod
@@ -417,7 +465,7 @@ class HipKernels:
             self._sample_ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=logits.device)
         self._check(self.lib.lev_sample(_ptr(logits), _rows(logits, "sample: logits"), _ptr(temperatures), _ptr(keys),
                                         _ptr(positions), _ptr(out_tokens), _ptr(out_logprobs), _ptr(self._sample_ws), R, V,
-                                        _stream()))
+                                        self._s()))
 
 
 _KERNELS = None

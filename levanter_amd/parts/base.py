@@ -36,6 +36,8 @@ class AttentionMeta:
     n_decode: int
     max_kv_len: int  # the longest key range any token of the step reads
     _workspaces: Dict[Any, torch.Tensor] = field(default_factory=dict)
+    plans: Dict[Any, Any] = field(default_factory=dict)
+    """The kernel library's notes on this step (what it has checked and decided once for all layers of a cache group)."""
 
     def workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
         if nbytes <= 0:

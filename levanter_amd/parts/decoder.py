@@ -73,6 +73,16 @@ class DecoderLm:
 
     def forward(self, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
         """Run the step's tokens through the plan; float32 logits ``[len(logit_rows), vocab]``."""
+        hold = getattr(ctx.kernels, "hold_stream", None)
+        if hold is not None:
+            hold()  # hundreds of launches on the one current stream
+        try:
+            return self._forward(ctx, logit_rows)
+        finally:
+            if hold is not None:
+                ctx.kernels.release_stream()
+
+    def _forward(self, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
         x = self.embedding(ctx)
         for e in self.plan:
             block = self.blocks[e.layer]
