@@ -4,19 +4,31 @@
 // (hundreds to thousands of rows), where its tuned kernels are ahead of gemm_tile_kernel on most shapes, and only
 // with epilogues it has itself: bias, the tanh GELU ("gelu_new"), ReLU, and the residual as the C operand with beta = 1.
 // Everything else (other activations, shapes it has no kernel for) returns LEV_LIBRARY_UNSUPPORTED and the caller
-// runs the hand-written kernel. In the library's column-major terms the row-major problem is
+// runs the hand-written kernel. Which of the library's kernels runs a shape is not left to its heuristic alone: for
+// 256 rows and more the heuristic's candidates are timed once (its first choice is up to twice slower than its best on row
+// counts that are no multiple of the tile, 2,052 rows for instance) and row counts of one bucket of 64 share the result. In the library's column-major terms the row-major problem is
 //   D^T [N x M] = w_cm^T [N x K] . a_cm [K x M]  (+ C^T),  with w_cm = w seen as K x N (ld K), a_cm = a seen as K x M (ld lda),
 // so that the bias, one value per row of D^T, is the per-output-column bias of the row-major result.
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
+#include <chrono>
 
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "common.h"
 
 #define LEV_LIBRARY_UNSUPPORTED 1
 #define LEV_LIB_MAX_DEVICES 64
+#define LEV_LIB_CANDIDATES 16    // kernels asked of the heuristic for one shape
+#define LEV_LIB_TUNE_MIN_ROWS 256  // below, a product is bound by reading its weight and a timing loop over one weight
+                                   // (which then sits in the last-level cache) says nothing about the real step
+#define LEV_LIB_TUNE_RUNS 4
+#define LEV_LIB_ROW_BUCKET 64      // row counts up to the same multiple of this share one timing
 
 namespace {
 
@@ -26,6 +38,8 @@ struct Plan {
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   bool ok = false;
+  bool timed = false;  // the candidates have been timed on this shape and algo is the fastest of them
+  std::vector<hipblasLtMatmulHeuristicResult_t> candidates;  // in the heuristic's order; algo starts as the first
 };
 
 // (device, M, N, K, lda, ldr, ldo, epilogue, output dtype, residual?)
@@ -34,6 +48,11 @@ typedef std::tuple<int, int, int, int, long, long, long, int, int, int> PlanKey;
 std::mutex g_mutex;
 hipblasLtHandle_t g_handle[LEV_LIB_MAX_DEVICES];
 std::map<PlanKey, Plan> g_plans;
+// What timing chose, by PlanKey with the row count replaced by its bucket (rows_bucket): the library's index of the kernel.
+// Row counts of one bucket share it, so a serving run whose steps differ by a few rows times once, not once a row count.
+std::map<PlanKey, int> g_timed_index;
+
+int rows_bucket(int M) { return (M + LEV_LIB_ROW_BUCKET - 1) / LEV_LIB_ROW_BUCKET; }
 
 const char* status_name(hipblasStatus_t s) {
   switch (s) {
@@ -80,16 +99,100 @@ int make_plan(hipblasLtHandle_t handle, Plan* p, int M, int N, int K, long lda, 
   LIB_CHECK(hipblasLtMatmulPreferenceCreate(&pref));
   const uint64_t ws = max_workspace;
   hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-  hipblasLtMatmulHeuristicResult_t result[1];
+  hipblasLtMatmulHeuristicResult_t result[LEV_LIB_CANDIDATES];
   int found = 0;
   if (s == HIPBLAS_STATUS_SUCCESS)
-    s = hipblasLtMatmulAlgoGetHeuristic(handle, p->desc, p->lw, p->la, p->lc, p->ld, pref, 1, result, &found);
+    s = hipblasLtMatmulAlgoGetHeuristic(handle, p->desc, p->lw, p->la, p->lc, p->ld, pref, LEV_LIB_CANDIDATES, result, &found);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (s != HIPBLAS_STATUS_SUCCESS || found < 1) return LEV_LIBRARY_UNSUPPORTED;  // p->ok stays false: remembered, not asked again
-  p->algo = result[0].algo;
-  p->workspace = result[0].workspaceSize;
+  for (int i = 0; i < found; ++i)
+    if (result[i].state == HIPBLAS_STATUS_SUCCESS && result[i].workspaceSize <= max_workspace) p->candidates.push_back(result[i]);
+  if (p->candidates.empty()) return LEV_LIBRARY_UNSUPPORTED;
+  p->algo = p->candidates[0].algo;
+  p->workspace = p->candidates[0].workspaceSize;
   p->ok = true;
   return 0;
+}
+
+// 0: the heuristic's first kernel is taken; 1 (default): the candidates of a shape are timed at its first call outside a
+// stream capture and the fastest is kept; 2: the timings are printed as well.
+int tune_level() {
+  static const int level = [] {
+    const char* e = getenv("LEVANTER_AMD_GEMM_TUNE");
+    return e ? atoi(e) : 1;
+  }();
+  return level;
+}
+
+// Times every candidate of a plan on the call's own operands, writing to a buffer of its own (a product into the residual
+// stream adds to its output, so the real output cannot take repeated runs), and keeps the fastest. The heuristic's order is
+// a table look-up by size; on this chip its first kernel is often not the fastest one for the shape at hand.
+// Allocates and synchronises: called only outside a stream capture, once per shape and process.
+int time_candidates(hipblasLtHandle_t handle, Plan* p, const void* a, const void* w, const float* residual, void* workspace, int M,
+                     int N, long ldo, int out_dtype, hipStream_t stream) {
+  p->timed = true;
+  if (p->candidates.size() < 2) return -1;
+  auto t_begin = std::chrono::steady_clock::now();
+  const size_t bytes = (size_t)M * (size_t)ldo * (out_dtype == LEV_F32 ? 4 : 2);
+  void* scratch = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipMalloc(&scratch, bytes) != hipSuccess) { (void)hipGetLastError(); return -1; }
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    (void)hipGetLastError();
+    if (e0) (void)hipEventDestroy(e0);
+    (void)hipFree(scratch);
+    return -1;
+  }
+  const float alpha = 1.0f, beta = residual ? 1.0f : 0.0f;
+  const void* c = residual ? (const void*)residual : (const void*)scratch;
+  float best = -1.0f;
+  int best_i = 0;
+  for (size_t i = 0; i < p->candidates.size(); ++i) {
+    const hipblasLtMatmulHeuristicResult_t& cand = p->candidates[i];
+    bool ok = true;
+    float ms = 0.0f;
+    for (int run = 0; run <= LEV_LIB_TUNE_RUNS && ok; ++run) {  // run 0 loads the kernel and is not timed
+      if (run == 1) ok = hipEventRecord(e0, stream) == hipSuccess;
+      ok = ok && hipblasLtMatmul(handle, p->desc, &alpha, w, p->lw, a, p->la, &beta, c, p->lc, scratch, p->ld, &cand.algo, workspace,
+                                 cand.workspaceSize, stream) == HIPBLAS_STATUS_SUCCESS;
+    }
+    ok = ok && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    if (!ok) { (void)hipGetLastError(); (void)hipStreamSynchronize(stream); continue; }
+    if (tune_level() >= 2) {
+      hipblasLtMatmulAlgo_t algo = cand.algo;
+      fprintf(stderr, "linear (library) M=%d N=%d: candidate %zu (kernel %d) %.1f us\n", M, N, i, hipblaslt_ext::getIndexFromAlgo(algo),
+              ms * 1000.0f / LEV_LIB_TUNE_RUNS);
+    }
+    if (best < 0.0f || ms < best) { best = ms; best_i = (int)i; }
+  }
+  if (best >= 0.0f) {
+    p->algo = p->candidates[best_i].algo;
+    p->workspace = p->candidates[best_i].workspaceSize;
+    if (tune_level() >= 2)
+      fprintf(stderr, "linear (library) M=%d N=%d: kept candidate %d after %.1f ms\n", M, N, best_i,
+              std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t_begin).count());
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipStreamSynchronize(stream);
+  (void)hipFree(scratch);
+  return best >= 0.0f ? hipblaslt_ext::getIndexFromAlgo(p->algo) : -1;
+}
+
+// Gives a plan the kernel that timing chose for another row count of its bucket, if that kernel takes this problem too.
+bool adopt_index(hipblasLtHandle_t handle, Plan* p, int index, bool residual, size_t max_workspace) {
+  std::vector<int> indices(1, index);
+  std::vector<hipblasLtMatmulHeuristicResult_t> found;
+  if (hipblaslt_ext::getAlgosFromIndex(handle, indices, found) != HIPBLAS_STATUS_SUCCESS || found.empty()) return false;
+  const float alpha = 1.0f, beta = residual ? 1.0f : 0.0f;
+  size_t need = 0;
+  if (hipblaslt_ext::matmulIsAlgoSupported(handle, p->desc, &alpha, p->lw, p->la, &beta, p->lc, p->ld, found[0].algo, need) !=
+          HIPBLAS_STATUS_SUCCESS || need > max_workspace)
+    return false;
+  p->algo = found[0].algo;
+  p->workspace = need;
+  return true;
 }
 
 }  // namespace
@@ -109,35 +212,43 @@ extern "C" int lev_linear_library(const void* a, long lda, const void* w, const 
   if (epilogue_of(act, bias != nullptr, &epilogue)) return LEV_LIBRARY_UNSUPPORTED;
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LEV_LIB_MAX_DEVICES) return lev_fail("linear (library): no current device");
-  Plan plan;
-  hipblasLtHandle_t handle;
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (!g_handle[dev]) LIB_CHECK(hipblasLtCreate(&g_handle[dev]));
-    handle = g_handle[dev];
-    const PlanKey key(dev, M, N, K, lda, residual ? ldr : 0, ldo, (int)epilogue, out_dtype, residual ? 1 : 0);
-    auto it = g_plans.find(key);
-    if (it == g_plans.end()) {
-      Plan p;
-      const int rc = make_plan(handle, &p, M, N, K, lda, ldr, ldo, epilogue, bias != nullptr, residual != nullptr,
-                               out_dtype == LEV_F32 ? HIP_R_32F : HIP_R_16BF, (size_t)workspace_bytes);
-      if (rc < 0) return rc;
-      it = g_plans.emplace(key, p).first;
-    }
-    plan = it->second;
+  // One lock for the look-up, the bias pointer (the descriptor is shared by every call of this shape) and the launch.
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!g_handle[dev]) LIB_CHECK(hipblasLtCreate(&g_handle[dev]));
+  hipblasLtHandle_t handle = g_handle[dev];
+  const PlanKey key(dev, M, N, K, lda, residual ? ldr : 0, ldo, (int)epilogue, out_dtype, residual ? 1 : 0);
+  auto it = g_plans.find(key);
+  if (it == g_plans.end()) {
+    Plan p;
+    const int rc = make_plan(handle, &p, M, N, K, lda, ldr, ldo, epilogue, bias != nullptr, residual != nullptr,
+                             out_dtype == LEV_F32 ? HIP_R_32F : HIP_R_16BF, (size_t)workspace_bytes);
+    if (rc < 0) return rc;
+    it = g_plans.emplace(key, p).first;
   }
+  Plan& plan = it->second;
   if (!plan.ok) return LEV_LIBRARY_UNSUPPORTED;
-  if (plan.workspace > (size_t)workspace_bytes || (plan.workspace > 0 && !workspace))
-    return lev_fail("linear (library): the chosen kernel needs %zu bytes of workspace, %ld were brought", plan.workspace, workspace_bytes);
-  if (bias) {  // the descriptor is shared by every call of this shape: the pointer is set under the lock, with the launch
-    std::lock_guard<std::mutex> lock(g_mutex);
+  if (bias) {
     const void* bp = bias;
     LIB_CHECK(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp)));
-    const float alpha = 1.0f, beta = residual ? 1.0f : 0.0f;
-    LIB_CHECK(hipblasLtMatmul(handle, plan.desc, &alpha, w, plan.lw, a, plan.la, &beta, residual ? (const void*)residual : (const void*)out,
-                              plan.lc, out, plan.ld, &plan.algo, workspace, plan.workspace, stream));
-    return 0;
   }
+  if (!plan.timed && M >= LEV_LIB_TUNE_MIN_ROWS && tune_level() >= 1) {
+    const PlanKey bucket(dev, rows_bucket(M), N, K, lda, residual ? ldr : 0, ldo, (int)epilogue, out_dtype, residual ? 1 : 0);
+    auto known = g_timed_index.find(bucket);
+    if (known != g_timed_index.end()) {
+      plan.timed = true;  // whether it fits or not: the plan is settled
+      const bool fits = known->second >= 0 && adopt_index(handle, &plan, known->second, residual != nullptr, (size_t)workspace_bytes);
+      if (tune_level() >= 2)
+        fprintf(stderr, "linear (library) M=%d N=%d K=%d: kernel %d of its bucket %s\n", M, N, K, known->second,
+                fits ? "taken" : "does not fit");
+    } else {
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) { (void)hipGetLastError(); capturing = hipStreamCaptureStatusActive; }
+      if (capturing == hipStreamCaptureStatusNone)
+        g_timed_index[bucket] = time_candidates(handle, &plan, a, w, residual, workspace, M, N, ldo, out_dtype, stream);
+    }
+  }
+  if (plan.workspace > 0 && !workspace)
+    return lev_fail("linear (library): the chosen kernel needs %zu bytes of workspace, none was brought", plan.workspace);
   const float alpha = 1.0f, beta = residual ? 1.0f : 0.0f;
   LIB_CHECK(hipblasLtMatmul(handle, plan.desc, &alpha, w, plan.lw, a, plan.la, &beta, residual ? (const void*)residual : (const void*)out,
                             plan.lc, out, plan.ld, &plan.algo, workspace, plan.workspace, stream));

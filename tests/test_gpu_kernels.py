@@ -253,6 +253,28 @@ def test_linear_bf16_prompt_sized_rows_with_and_without_the_vendor_library(K, li
         assert n_library == 6 and len(calls) == 6 and all(rc == 0 for rc in calls), calls  # the library took all but the last
 
 
+def test_row_counts_of_one_bucket_share_the_kernel_that_timing_chose(K, monkeypatch):
+    """From 256 rows the library's candidates for a shape are timed at its first call, on an output of their own (the
+    product into the residual stream adds to its output: timing on the real one would add several times), and row counts
+    up to the same multiple of 64 take the kernel chosen then. Every one of them is the product, in place too."""
+    monkeypatch.setattr(K, "use_library", lambda M, N, K_, act: True)
+    K_, N = 2056, 3080
+    w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=1).to(DEV)
+    bias = _rand(N, seed=2).to(DEV)
+    for M in (1000, 990, 961, 1024, 1001):  # 1000 is timed; 990, 961 and 1001 follow it; 1024 belongs to the same bucket as well
+        a = _rand(M, K_, dtype=torch.bfloat16, seed=M).to(DEV)
+        x = _rand(M, N, seed=M + 1).to(DEV)
+        want = x.double() + a.double() @ w.double().t() + bias.double()
+        for _ in range(2):  # the call that times and the call after it give the same
+            out = x.clone()
+            K.linear(a, w, bias, out, residual=out)
+            assert float((out.double() - want).abs().max() / want.abs().max()) < 2e-3, M
+        h = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+        K.linear(a, w, None, h, activation="gelu_new")
+        want = torch.nn.functional.gelu(a.double() @ w.double().t(), approximate="tanh")
+        assert float((h.double() - want).abs().max() / want.abs().max()) < 2e-2, M
+
+
 @pytest.mark.parametrize("M,K_,N,rows", [(64, 4096, 4096, None), (100, 16384, 4096, [99, 3, 3, 50]), (33, 8192, 1608, None),
                                          (300, 6400, 1600, [299, 0]), (64, 4096, 4104, None), (40, 8192, 8200, None)])
 def test_a_product_that_leaves_its_ranges_to_the_norm(K, M, K_, N, rows):
