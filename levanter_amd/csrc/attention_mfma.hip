@@ -48,6 +48,27 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return float
 // key (0..63) of row i of score tile (u, h)
 __device__ __forceinline__ int tile_key(int u, int h, int i) { return 32 * u + 8 * (i >> 2) + 4 * h + (i & 3); }
 
+// Eight consecutive keys' values of one dimension (two to a word) with all but the first n made zero. A key beyond the
+// range has a probability of zero, but what its slot of the cache holds may be anything, NaN too (a page is not cleared
+// when it is given to another request), and zero times that would reach the sum.
+__device__ __forceinline__ u32x4 first_keys_mask(int n) {
+  u32x4 mk;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) mk[e] = n >= 2 * e + 2 ? 0xffffffffu : (n == 2 * e + 1 ? 0x0000ffffu : 0u);
+  return mk;
+}
+
+// The largest of the values that lanes l, l ^ 16, l ^ 32 and l ^ 48 hold, in all four of them. The two swaps are vector
+// ALU instructions of their own on this chip; the same through ds_bpermute costs two round trips to the LDS, one after the
+// other, in the middle of the softmax's chain of dependent steps.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+  const u32x2_t a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);  // {lower half twice, upper half twice}
+  const float w = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const u32x2_t b = __builtin_amdgcn_permlane16_swap(__float_as_uint(w), __float_as_uint(w), false, false);  // {rows 0 0 2 2, rows 1 1 3 3}
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 // One block of 64 keys for one wave: scores are in st[u][h] (S^T tiles, raw dot products).
 // Applies scale and mask, updates the running max m and sum l (per lane: column = query row),
 // rescales the output accumulators and returns the probabilities as B operands pf[u].
@@ -82,8 +103,7 @@ __device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale_log2, 
           mx = fmaxf(mx, s);
         }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = max_over_lane_groups(mx);
   const float m_new = fmaxf(m, mx);
   const float base = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
   const float corr = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - base);
@@ -111,22 +131,76 @@ __device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale_log2, 
                   pack_bf16(p[u][1][2], p[u][1][3])};
 }
 
+// The softmax of a block that needs no mask, in two parts so that the products of the next block can be issued between
+// them. The running maximum is only raised (and sum and outputs rescaled) when a block's maximum exceeds it by more than
+// LAZY_MAX in the base-2 domain: probabilities then reach 2^LAZY_MAX at most, which costs the 32-bit sums nothing, and
+// the 4 * NDT multiplications of the rescaling leave nearly every block. m, l and o mean what they mean to softmax_block
+// (which takes any m that bounds nothing: it only needs sum and outputs to be scaled by the same exp2(-m)).
+#define LAZY_MAX 8.0f
+// Part one: is any row's maximum to be raised? (Wave-uniform answer.) m_cand is the lane's candidate.
+__device__ __forceinline__ bool softmax_interior_max(const f32x4 st[2][2], float scale_log2, float m, float& m_cand) {
+  float mx = fmaxf(fmaxf(st[0][0][0], st[0][0][1]), fmaxf(st[0][0][2], st[0][0][3]));
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      if (u + h > 0) mx = fmaxf(mx, fmaxf(fmaxf(st[u][h][0], st[u][h][1]), fmaxf(st[u][h][2], st[u][h][3])));
+  m_cand = max_over_lane_groups(mx) * scale_log2;  // the scale is positive: the largest raw score is the largest score
+  return __builtin_amdgcn_ballot_w64(m_cand > m + LAZY_MAX) != 0;
+}
+__device__ __forceinline__ void softmax_interior_raise(float m_cand, float& m, float& l, f32x4* o) {
+  const float m_new = fmaxf(m, m_cand);
+  const float corr = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+  l *= corr;
+  m = m_new;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t) {
+    o[t][0] *= corr; o[t][1] *= corr; o[t][2] *= corr; o[t][3] *= corr;
+  }
+}
+// Part two: probabilities (scale and maximum in one multiply-add under the exponential), their sum, and the B operands.
+__device__ __forceinline__ void softmax_interior_exp(const f32x4 st[2][2], float scale_log2, float m, float& l, u32x4 pf[2]) {
+  float p[2][2][4];
+  float psum = 0.f;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        p[u][h][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[u][h][r], scale_log2, -m));
+        psum += p[u][h][r];
+      }
+  l += psum;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+    pf[u] = u32x4{pack_bf16(p[u][0][0], p[u][0][1]), pack_bf16(p[u][0][2], p[u][0][3]), pack_bf16(p[u][1][0], p[u][1][1]),
+                  pack_bf16(p[u][1][2], p[u][1][3])};
+}
+
 // ------------------------------------------------------------------------------------------------
 // Prefill: a workgroup of PF_WAVES waves per (tile of up to PF_ROWS consecutive query tokens, head). Each wave
-// owns PF_QT tiles of 16 query rows: a key or value fragment read from LDS feeds PF_QT products, which is what
-// keeps the kernel off the LDS bandwidth limit. Blocks of 64 keys go global -> registers -> LDS; the loads of
-// the next block are in flight during the products (barriers order LDS only).
+// owns PF_QT tiles of 16 query rows. Blocks of 64 keys go global -> registers -> LDS, keys and values in two LDS
+// buffers each, and the loop is skewed: in the iteration of block kb a wave
+//   multiplies the scores of block kb + 1 (matrix pipe, key fragments from LDS),
+//   takes the softmax of block kb's scores, which the iteration before left in registers (vector ALU),
+//   stages the keys of block kb + 2 and the values of block kb + 1 and requests those after them,
+//   multiplies block kb's probabilities with its values (matrix pipe, value fragments from LDS).
+// The two products of a block no longer wait for its softmax between them, so that the matrix pipe, the LDS and the
+// vector ALU of a wave work at the same time; one barrier an iteration orders the LDS buffers. (With both products and
+// the softmax of one block in one iteration, between two barriers, all waves of a CU are in the same phase at the same
+// time and each phase waits for another unit: 91 us a layer for a 2,048-token prompt of 32 heads of 128.)
 #include "attention_config.h"
 
-typedef bf16_t (*KsPtr)[NCHUNK][16][8];
-typedef bf16_t (*VsPtr)[VS_STRIDE];
+typedef bf16_t (*KsPtr)[4][NCHUNK][16][8];  // [buffer][score tile 2u+h][chunk][row][8]
+typedef bf16_t (*VsPtr)[HD][VS_STRIDE];     // [buffer][dim][key]
 
 __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
                                              const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                                              const int* __restrict__ positions, const int* __restrict__ token_seq,
                                              const int* __restrict__ block_tables, int bt_stride, int t0, int rows, int h,
                                              int H, int KVH, int ps_shift, float scale, int window, KsPtr Ks, VsPtr Vs) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int fr = lane & 15, g = lane >> 4;
   const int kvh = h / (H / KVH);
   const float scale_log2 = scale * 1.4426950408889634f;
@@ -161,107 +235,76 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
     for (int t = 0; t < NDT; ++t) o[qt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  // What a thread moves of a block: of K the 16-byte chunks c = wave, wave + PF_WAVES, .. of ONE key (tid % 64); of V
+  // 8 consecutive keys of one dimension per chunk. Everything but the page and the block's first key is fixed per thread.
   constexpr int KCH = (64 * NCHUNK + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks of K per thread and block
   constexpr int VCH = (HD * 8 + PF_THREADS - 1) / PF_THREADS;
-  // two register sets: block kb + 2 is loaded while block kb is multiplied (a load has two iterations to arrive)
-  u32x4 kr[2][KCH], vr[2][VCH];
-  bool kok[2][KCH], vok[2][VCH];  // does the chunk hold keys of the range (decided when it is loaded, used when it is staged)
-  const int PS = 1 << ps_shift, ps_mask = PS - 1;
+  static_assert(PF_THREADS % 64 == 0, "a thread's K chunks belong to one key");
+  // every thread has a chunk in every round (then staging has no branch, and the iteration below is one basic block)
+  constexpr bool K_EXACT = (64 * NCHUNK) % PF_THREADS == 0, V_EXACT = (HD * 8) % PF_THREADS == 0;
+  const int ps_mask = (1 << ps_shift) - 1;
   const size_t head_elems = (size_t)HD << ps_shift;
-  // The page ids of a block of 64 keys (at most 4 of them) are read one iteration before the block's data is
-  // requested, so that no data load waits for a table lookup. They are read with vector loads on purpose (the
-  // index is made opaque): scalar loads share a counter with LDS and, while one is in flight, the compiler
-  // waits for every LDS read at once instead of pipelining them.
-  constexpr int NPG = 4;
-  // pg[0..3]: the ids as loaded (not looked at until the next iteration, so nothing waits for the loads here);
-  // pg[4]: bit j says whether entry j exists
-  auto load_pages = [&](int kb, int pg[NPG + 1]) {
-    const int b0 = (kb * 64) >> ps_shift;
-    int valid = 0;
+  const size_t page_elems = (size_t)KVH * head_elems;
+  const int k_kk = tid & 63;
+  size_t k_coff[KCH];
 #pragma unroll
-    for (int j = 0; j < NPG; ++j) {
-      const int idx = b0 + j;
-      int at = min(idx, bt_stride - 1);
-      asm volatile("" : "+v"(at));
-      pg[j] = bt[at];
-      valid |= (idx < bt_stride && (j << ps_shift) < 64) ? (1 << j) : 0;
-    }
-    pg[NPG] = valid;
+  for (int i = 0; i < KCH; ++i) k_coff[i] = (size_t)kvh * head_elems + (((size_t)min((tid >> 6) + PF_WAVES * i, NCHUNK - 1) << ps_shift) * 8);
+  int v_kk[VCH];
+  size_t v_doff[VCH];
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    const int y = min(tid + PF_THREADS * i, HD * 8 - 1);
+    const int j = y / (HD * 2), rem = y % (HD * 2);
+    v_kk[i] = 16 * j + 8 * (rem & 1);  // first of 8 keys; a page holds a multiple of 16
+    v_doff[i] = (size_t)kvh * head_elems + ((size_t)(rem >> 1) << ps_shift);
+  }
+  // Page ids are read an iteration before the data they lead to is requested, so that no data load waits for a table
+  // lookup. A key beyond the table's width is beyond `hi` as well and is zeroed when it is staged.
+  auto k_page_of = [&](int kb) { return bt[min((kb * 64 + k_kk) >> ps_shift, bt_stride - 1)]; };
+  auto v_pages_of = [&](int kb, int page[VCH]) {
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) page[i] = bt[min((kb * 64 + v_kk[i]) >> ps_shift, bt_stride - 1)];
   };
-  auto pick = [&](const int pg[NPG + 1], int j) {
-    const int v = j == 0 ? pg[0] : (j == 1 ? pg[1] : (j == 2 ? pg[2] : pg[3]));
-    return ((pg[NPG] >> j) & 1) ? v : -1;
-  };
+  u32x4 kr[KCH], vr[VCH];
+  // Values beyond the key range are zeroed when they are staged (decided when they are loaded). Keys are staged as they
+  // come: a score is looked at only behind the mask, which selects and does not add.
+  int vkeep[VCH];  // how many of the chunk's 8 keys are kept
   // Loads are unconditional (a chunk outside the key range reads page 0 and is zeroed when it is staged):
   // conditional loads would make the compiler wait for them at the join instead of after the products.
-  auto prefetch = [&](int set, int kb, const int pg[NPG + 1]) {
-    const int key0 = kb * 64;
+  auto load_k = [&](int kb, int page) {
+    const int kp = kb * 64 + k_kk;
+    const bf16_t* base = k_pages + (size_t)max(page, 0) * page_elems + (size_t)(kp & ps_mask) * 8;
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int x = tid + PF_THREADS * i;
-      const int kk = x & 63, c = min(x >> 6, NCHUNK - 1);
-      const int kp = key0 + kk;
-      const int page = pick(pg, kk >> ps_shift);
-      kok[set][i] = kp <= hi && kp >= lo_tile && page >= 0;
-      kr[set][i] = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + (((size_t)c << ps_shift) + (kp & ps_mask)) * 8);
-    }
+    for (int i = 0; i < KCH; ++i) kr[i] = *reinterpret_cast<const u32x4*>(base + k_coff[i]);
+  };
+  auto load_v = [&](int kb, const int page[VCH]) {
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int y = min(tid + PF_THREADS * i, HD * 8 - 1);
-      const int j = y / (HD * 2), rem = y % (HD * 2);
-      const int d = rem >> 1, half = rem & 1;
-      const int kk = 16 * j + 8 * half;  // first of 8 keys; a page holds a multiple of 16
-      const int kp = key0 + kk;
-      const int page = pick(pg, kk >> ps_shift);
-      vok[set][i] = kp <= hi && kp + 7 >= lo_tile && page >= 0;
-      vr[set][i] = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + ((size_t)d << ps_shift) + (kp & ps_mask));
+      const int kp = kb * 64 + v_kk[i];
+      vkeep[i] = (kp + 7 >= lo_tile && page[i] >= 0) ? hi - kp + 1 : 0;
+      vr[i] = *reinterpret_cast<const u32x4*>(v_pages + (size_t)max(page[i], 0) * page_elems + v_doff[i] + (kp & ps_mask));
     }
   };
-  auto stage = [&](int set) {
+  auto stage_k = [&](int buf) {
+    const int tile = 2 * (k_kk >> 5) + ((k_kk & 7) >> 2);
+    const int row = 4 * ((k_kk & 31) >> 3) + (k_kk & 3);
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int x = tid + PF_THREADS * i;
-      const int kk = x & 63, c = x >> 6;
-      if (c < NCHUNK) {
-        const int tile = 2 * (kk >> 5) + ((kk & 7) >> 2);
-        const int row = 4 * ((kk & 31) >> 3) + (kk & 3);
-        *reinterpret_cast<u32x4*>(&Ks[tile][c][row][0]) = kok[set][i] ? kr[set][i] : u32x4{0, 0, 0, 0};
-      }
+      const int c = (tid >> 6) + PF_WAVES * i;
+      if (K_EXACT || c < NCHUNK) *reinterpret_cast<u32x4*>(&Ks[buf][tile][c][row][0]) = kr[i];
     }
+  };
+  auto stage_v = [&](int buf, bool whole) {  // whole: the block lies in the key range, nothing to zero
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
       const int y = tid + PF_THREADS * i;
-      if (y < HD * 8) {
-        const int j = y / (HD * 2), rem = y % (HD * 2);
-        *reinterpret_cast<u32x4*>(&Vs[rem >> 1][16 * j + 8 * (rem & 1)]) = vok[set][i] ? vr[set][i] : u32x4{0, 0, 0, 0};
-      }
+      if (V_EXACT || y < HD * 8)
+        *reinterpret_cast<u32x4*>(&Vs[buf][(y % (HD * 2)) >> 1][v_kk[i]]) = whole ? vr[i] : (vr[i] & first_keys_mask(vkeep[i]));
     }
   };
-
-  const int kb_first = lo_tile / 64, kb_last = hi / 64;
   const int n_qt = min(PF_QT, max(0, (rows - wave_row0 + 15) / 16));  // query tiles of this wave that hold rows
-  int pgs[2][NPG + 1];  // page ids of the blocks with even / odd distance from the first
-  load_pages(kb_first, pgs[0]);
-  load_pages(kb_first + 1, pgs[1]);
-  prefetch(0, kb_first, pgs[0]);
-  prefetch(1, kb_first + 1, pgs[1]);
-  load_pages(kb_first + 2, pgs[0]);
-  auto block = [&](int kb, int set) {
-    lds_barrier();  // everyone has finished reading the previous block
-    stage(set);
-    lds_barrier();
-    load_pages(kb + 3, pgs[set ^ 1]);  // older than the data loads below: waiting for them later leaves those in flight
-    prefetch(set, kb + 2, pgs[set]);   // blocks past the last one are masked by their key positions
-    const int key0 = kb * 64;
-    bool live[PF_QT];  // does query tile qt see any key of this block (wave-uniform)
-    bool any = false;
-#pragma unroll
-    for (int qt = 0; qt < PF_QT; ++qt) {
-      live[qt] = qt < n_qt && key0 <= pos0 + wave_row0 + qt * 16 + 15;
-      any = any || live[qt];
-    }
-    if (!any) return;
-    f32x4 st[PF_QT][2][2];
+  // scores of a block for the query tiles that see it (live, wave-uniform), from the keys in Ks[buf]
+  auto scores = [&](int buf, const bool live[PF_QT], f32x4 st[PF_QT][2][2]) {
 #pragma unroll
     for (int qt = 0; qt < PF_QT; ++qt)
 #pragma unroll
@@ -275,36 +318,160 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
           const int c = 4 * s + g;
-          const u32x4 kf = c < NCHUNK ? *reinterpret_cast<const u32x4*>(&Ks[2 * u + hh][c][fr][0]) : u32x4{0, 0, 0, 0};
+          const u32x4 kf = c < NCHUNK ? *reinterpret_cast<const u32x4*>(&Ks[buf][2 * u + hh][c][fr][0]) : u32x4{0, 0, 0, 0};
 #pragma unroll
           for (int qt = 0; qt < PF_QT; ++qt)
             if (live[qt])
               st[qt][u][hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[qt][s]), st[qt][u][hh], 0, 0, 0);
         }
-    u32x4 pf[PF_QT][2];
-#pragma unroll
-    for (int qt = 0; qt < PF_QT; ++qt)
-      if (live[qt]) {
-        const int p0 = pos0 + wave_row0 + qt * 16;  // first row of the tile: does it see the whole block, and the last row too
-        const bool need_mask = !(key0 + 63 <= p0 && (window <= 0 || p0 + 15 - window + 1 <= key0));
-        softmax_block(st[qt], scale_log2, q_pos[qt], lo[qt], key0, g, need_mask, m[qt], l[qt], o[qt], pf[qt]);
-      }
+  };
+  auto values = [&](int buf, const bool live[PF_QT], const u32x4 pf[PF_QT][2]) {
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vs[16 * t + fr][32 * u + 8 * g]);
+        const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vs[buf][16 * t + fr][32 * u + 8 * g]);
 #pragma unroll
         for (int qt = 0; qt < PF_QT; ++qt)
           if (live[qt]) o[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[qt][u]), o[qt][t], 0, 0, 0);
       }
   };
+  auto live_tiles = [&](int kb, bool live[PF_QT]) {  // which query tiles see any key of block kb
+    bool any = false;
+#pragma unroll
+    for (int qt = 0; qt < PF_QT; ++qt) {
+      live[qt] = qt < n_qt && kb * 64 <= pos0 + wave_row0 + qt * 16 + 15;
+      any = any || live[qt];
+    }
+    return any;
+  };
+
+  const int kb_first = lo_tile / 64, kb_last = hi / 64;
+  int kpage, vpage[VCH];
+  f32x4 st[PF_QT][2][2];  // raw scores of the block whose softmax comes next
+  bool live[PF_QT];
+  // Before the loop: K and V of the first block are staged, K of the second, and the scores of the first are taken;
+  // K of the third block and V of the second are on their way, the page ids after them are read.
+  kpage = k_page_of(kb_first);
+  v_pages_of(kb_first, vpage);
+  load_k(kb_first, kpage);
+  load_v(kb_first, vpage);
+  kpage = k_page_of(kb_first + 1);
+  v_pages_of(kb_first + 1, vpage);
+  lds_barrier();  // a tile before this one (the other of a pair) has been read to its end
+  stage_k(0);
+  stage_v(0, false);
+  load_k(kb_first + 1, kpage);
+  load_v(kb_first + 1, vpage);
+  kpage = k_page_of(kb_first + 2);
+  v_pages_of(kb_first + 2, vpage);
+  stage_k(1);
+  load_k(kb_first + 2, kpage);
+  kpage = k_page_of(kb_first + 3);
+  lds_barrier();
+  if (live_tiles(kb_first, live)) scores(0, live, st);
+
+  // Iteration of block kb. Ks[cur ^ 1] holds the keys of kb + 1, Vs[cur] the values of kb; kr holds the keys of kb + 2,
+  // vr the values of kb + 1 (requested an iteration ago); kpage / vpage are the pages of K(kb + 3) / V(kb + 2).
+  auto iteration = [&](int kb, int cur) {
+    lds_barrier();  // everyone has staged what this iteration reads and has read what it overwrites
+    const int key0 = kb * 64;
+    // Every row of the wave sees every key of this block (then it sees some of the next one too) and the values staged
+    // now lie in the key range: no branch between the parts of the iteration but the rare one that raises the maxima,
+    // and an order of issue given to the compiler. Left alone it emits each part by itself, every product behind a wait
+    // for its own LDS read.
+    const int p_first = pos0 + wave_row0, p_last = p_first + (PF_QT - 1) * 16 + 15;
+    if (n_qt == PF_QT && key0 + 63 <= p_first && (window <= 0 || p_last - window + 1 <= key0) && key0 + 127 <= hi) {
+      bool all[PF_QT];
+      float m_cand[PF_QT];
+      bool raise = false;
+#pragma unroll
+      for (int qt = 0; qt < PF_QT; ++qt) {
+        all[qt] = true;
+        raise = softmax_interior_max(st[qt], scale_log2, m[qt], m_cand[qt]) || raise;
+      }
+      if (raise) {
+#pragma unroll
+        for (int qt = 0; qt < PF_QT; ++qt) softmax_interior_raise(m_cand[qt], m[qt], l[qt], o[qt]);
+      }
+      f32x4 st_next[PF_QT][2][2];
+      u32x4 pf[PF_QT][2];
+      scores(cur ^ 1, all, st_next);
+#pragma unroll
+      for (int qt = 0; qt < PF_QT; ++qt) softmax_interior_exp(st[qt], scale_log2, m[qt], l[qt], pf[qt]);
+      stage_k(cur);
+      stage_v(cur ^ 1, true);
+      load_k(kb + 3, kpage);
+      load_v(kb + 2, vpage);
+      kpage = k_page_of(kb + 4);
+      v_pages_of(kb + 3, vpage);
+      values(cur, all, pf);
+#pragma unroll
+      for (int qt = 0; qt < PF_QT; ++qt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh) st[qt][u][hh] = st_next[qt][u][hh];
+      // the score products with their key fragments spread over the exponentials ...
+      constexpr int N_QK = 4 * NKS * PF_QT, N_KF = 4 * NKS, N_PV = 2 * NDT * PF_QT, N_VF = 2 * NDT;
+      constexpr int EXP_VALU = 64 * PF_QT;
+      constexpr int AHEAD = 6;  // LDS reads issued before the first product
+      __builtin_amdgcn_sched_group_barrier(0x100, AHEAD < N_KF ? AHEAD : N_KF, 0);
+#pragma unroll
+      for (int i = 0; i < N_QK; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i * N_KF / N_QK + AHEAD < N_KF && (i * N_KF) % N_QK < N_KF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (EXP_VALU + N_QK - 1) / N_QK, 0);
+      }
+      // ... and the value products with theirs over the staging and the next requests
+      __builtin_amdgcn_sched_group_barrier(0x100, AHEAD < N_VF ? AHEAD : N_VF, 0);
+#pragma unroll
+      for (int i = 0; i < N_PV; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i * N_VF / N_PV + AHEAD < N_VF && (i * N_VF) % N_PV < N_VF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        if (i < KCH + VCH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        else if (i < 2 * (KCH + VCH) + 1 + VCH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      return;
+    }
+    bool live_next[PF_QT];
+    const bool any = live_tiles(kb, live);
+    const bool any_next = kb < kb_last && live_tiles(kb + 1, live_next);
+    f32x4 st_next[PF_QT][2][2];
+    u32x4 pf[PF_QT][2];
+    if (any_next) scores(cur ^ 1, live_next, st_next);
+    if (any) {
+#pragma unroll
+      for (int qt = 0; qt < PF_QT; ++qt)
+        if (live[qt]) {
+          const int p0 = pos0 + wave_row0 + qt * 16;  // first row of the tile: does it see the whole block, and the last row too
+          const bool need_mask = !(key0 + 63 <= p0 && (window <= 0 || p0 + 15 - window + 1 <= key0));
+          softmax_block(st[qt], scale_log2, q_pos[qt], lo[qt], key0, g, need_mask, m[qt], l[qt], o[qt], pf[qt]);
+        }
+    }
+    stage_k(cur);              // K(kb + 2) over K(kb), which the iteration before read
+    stage_v(cur ^ 1, false);   // V(kb + 1) over V(kb - 1)
+    load_k(kb + 3, kpage);  // blocks past the last one are zeroed by their key positions
+    load_v(kb + 2, vpage);
+    kpage = k_page_of(kb + 4);
+    v_pages_of(kb + 3, vpage);
+    if (any) values(cur, live, pf);
+    if (any_next) {
+#pragma unroll
+      for (int qt = 0; qt < PF_QT; ++qt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh) st[qt][u][hh] = st_next[qt][u][hh];
+    }
+  };
   int kb = kb_first;
   for (; kb + 1 <= kb_last; kb += 2) {
-    block(kb, 0);
-    block(kb + 1, 1);
+    iteration(kb, 0);
+    iteration(kb + 1, 1);
   }
-  if (kb <= kb_last) block(kb, 0);
+  if (kb <= kb_last) iteration(kb, 0);
 #pragma unroll
   for (int qt = 0; qt < PF_QT; ++qt) {
     float lq = l[qt];
@@ -330,14 +497,28 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
                           const int* __restrict__ positions, const int* __restrict__ token_seq,
                           const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int n_tiles, int pair,
                           int H, int KVH, int ps_shift, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[4][NCHUNK][16][8];  // [score tile 2u+h][chunk][row][8]
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[HD][VS_STRIDE];
-  const int first = blockIdx.x, second = n_tiles - 1 - blockIdx.x;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][4][NCHUNK][16][8];  // [buffer][score tile 2u+h][chunk][row][8]
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][VS_STRIDE];
+  // Workgroups go to the 8 XCDs in turn, each with an L2 of its own. A kv head's keys and values are read by every tile
+  // of every query head that shares it: all of those run on one XCD (kv head % 8), so that the cache is fetched from
+  // memory about once and not once per XCD (a 2,048-token prompt of 32 heads of 128: 34 MB a layer against 285 MB).
+  const int n_x = gridDim.x / H;  // tiles, or pairs of tiles
+  int x, h;
+  if (KVH % 8 == 0) {
+    const int xcd = blockIdx.x % 8, j = blockIdx.x / 8, G = H / KVH;
+    const int kvh = xcd + 8 * (j % (KVH / 8)), rest = j / (KVH / 8);  // rest counts (query head of the group, tile)
+    h = kvh * G + rest % G;
+    x = rest / G;
+  } else {
+    x = blockIdx.x % n_x;
+    h = blockIdx.x / n_x;
+  }
+  const int first = x, second = n_tiles - 1 - x;
   prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * first],
-               tiles[2 * first + 1], blockIdx.y, H, KVH, ps_shift, scale, window, Ks, Vs);
+               tiles[2 * first + 1], h, H, KVH, ps_shift, scale, window, Ks, Vs);
   if (pair && second > first)
     prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * second],
-                 tiles[2 * second + 1], blockIdx.y, H, KVH, ps_shift, scale, window, Ks, Vs);
+                 tiles[2 * second + 1], h, H, KVH, ps_shift, scale, window, Ks, Vs);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -466,12 +647,12 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
       }
     // value operands: tile dt, row fr is head dim 16*dt + fr, k-slots are keys 32u + 8g .. +7
     u32x4 vf[NDT][2];
-    uint32_t v_mask[2];
+    u32x4 v_mask[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int kp = key0 + 32 * u + 8 * g;
       const int page = vpg[u];
-      v_mask[u] = (kp <= pos && kp + 7 >= lo && page >= 0) ? 0xffffffffu : 0u;
+      v_mask[u] = first_keys_mask((kp + 7 >= lo && page >= 0) ? pos - kp + 1 : 0);
       const bf16_t* base = v_pages + ((size_t)max(page, 0) * KVH + kvh) * head_elems + (kp & ps_mask);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) vf[dt][u] = *reinterpret_cast<const u32x4*>(base + (size_t)(16 * dt + fr) * PS);
@@ -497,7 +678,7 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
       const int shift = (jn & 1) ? 16 : 0;
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
-        u32x4 v = vf[dt][u] & u32x4{v_mask[u], v_mask[u], v_mask[u], v_mask[u]};
+        u32x4 v = vf[dt][u] & v_mask[u];
         const uint32_t nvd = (nv2[dt / 2] >> (16 * (dt & 1))) & 0xffffu;
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = (has_new && w == e) ? ((v[e] & keep) | (nvd << shift)) : v[e];
@@ -626,7 +807,7 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
   if (n_prefill_tiles > 0) {
     // pairing halves the number of workgroups: only when every CU (256 of them) still gets one
     const int pair = (long)n_prefill_tiles * H >= 512;
-    dim3 grid(pair ? (n_prefill_tiles + 1) / 2 : n_prefill_tiles, H);
+    dim3 grid((pair ? (n_prefill_tiles + 1) / 2 : n_prefill_tiles) * H);
     LEV_NAME(attn_prefill_hd)<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
                                                         (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq,
                                                         block_tables, bt_stride, prefill_tiles, n_prefill_tiles, pair, H,

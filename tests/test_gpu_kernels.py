@@ -411,11 +411,13 @@ def test_linear_refuses_bad_sizes(K):
 
 
 def _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed):
-    """Random keys and values per request, written through the kv_write kernel into shuffled pages."""
+    """Random keys and values per request, written through the kv_write kernel into shuffled pages. What no request has
+    written holds NaN (a pool is not cleared between requests, and whatever a page held before is still there): a kernel
+    that lets an unwritten key or value reach a sum, even times a probability of zero, shows it in every output."""
     bt = random_block_tables(kv_lens, PS, n_pages, seed, "cpu")
     elems = KVH * HD * PS
-    kp = torch.zeros(n_pages, elems, dtype=dtype)
-    vp = torch.zeros(n_pages, elems, dtype=dtype)
+    kp = torch.full((n_pages, elems), float("nan"), dtype=dtype)
+    vp = torch.full((n_pages, elems), float("nan"), dtype=dtype)
     kd, vd = kp.to(DEV), vp.to(DEV)
     ks, vs = [], []
     for s, n in enumerate(kv_lens):
@@ -426,8 +428,8 @@ def _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed):
         K.kv_write(k.to(DEV), v.to(DEV), kd, vd, dest.to(DEV), KVH, HD, PS)
         ks.append(k)
         vs.append(v)
-    torch.testing.assert_close(kd.cpu(), kp, rtol=0, atol=0)
-    torch.testing.assert_close(vd.cpu(), vp, rtol=0, atol=0)
+    torch.testing.assert_close(kd.cpu(), kp, rtol=0, atol=0, equal_nan=True)
+    torch.testing.assert_close(vd.cpu(), vp, rtol=0, atol=0, equal_nan=True)
     return bt, kp, vp, kd, vd, ks, vs
 
 
@@ -446,6 +448,11 @@ ATTN_CASES = [
     (2, 2, 256, 16, [(1, 40), (9, 33)], None),
     (32, 32, 128, 16, [(1, 1850)], None),  # a lone long request: many key ranges, merged by the combine kernel
     (6, 2, 64, 16, [(1, 1200), (1, 520)], 600),
+    # prompts long enough that most key blocks of a tile lie wholly before its rows (the loop's branch-free iteration),
+    # alone, as a later portion, under a wide window, and at a head size whose staging leaves some threads without a chunk
+    (2, 2, 128, 16, [(300, 300)], None),
+    (4, 2, 64, 32, [(200, 456), (1, 30)], 300),
+    (3, 1, 96, 16, [(257, 700), (130, 130)], None),
 ]
 
 
@@ -522,6 +529,32 @@ def test_paged_attention_random_cases(K):
         want = torch.empty(T, H * HD, dtype=dtype)
         EMU.paged_attention(q, want, kp, vp, make_meta(runs, "cpu"), block_tables=bt, **args)
         torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2, msg=lambda m: case + "\n" + m)
+
+
+@pytest.mark.parametrize("ramp", ["rising", "falling", "steps"])
+def test_prefill_attention_when_the_largest_score_keeps_moving(K, ramp):
+    """The prompt kernel raises a row's running maximum only when a block of keys exceeds it by a margin, and rescales sum and
+    outputs then. Keys whose length grows along the sequence raise every row's maximum block after block, by little and by
+    much; falling lengths never raise it after the first block; steps raise it rarely and far. All three are the softmax."""
+    H = KVH = 2
+    HD, PS, n = 128, 16, 520
+    dtype = torch.bfloat16
+    pos = torch.arange(n, dtype=torch.float32)
+    length = {"rising": 0.2 + pos / 60.0, "falling": 8.0 - pos / 70.0, "steps": 0.3 + 4.0 * (pos // 130)}[ramp]
+    k = (_rand(n, KVH * HD, dtype=torch.float32, seed=1).sign() * length[:, None]).to(dtype)  # |k| = length: q . k grows with it
+    v = _rand(n, KVH * HD, dtype=dtype, seed=2)
+    q = (_rand(n, H * HD, dtype=torch.float32, seed=3).abs() * k.float().sign()).to(dtype)  # every term of q . k is positive
+    bt = random_block_tables([n], PS, 40, 3, "cpu")
+    kp = torch.full((40, KVH * HD * PS), float("nan"), dtype=dtype)
+    vp = torch.full((40, KVH * HD * PS), float("nan"), dtype=dtype)
+    EMU.kv_write(k, v, kp, vp, torch.tensor(dest_for(bt, 0, range(n), PS), dtype=torch.int32), KVH, HD, PS)
+    runs = [(n, n)]
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=0.02, window=None)
+    want = torch.empty(n, H * HD, dtype=dtype)
+    EMU.paged_attention(q, want, kp, vp, make_meta(runs, "cpu"), block_tables=bt, **args)
+    got = torch.full((n, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q.to(DEV), got, kp.to(DEV), vp.to(DEV), make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
