@@ -186,12 +186,17 @@ def _random_requests(rng, vocab, max_pos, n):
     return reqs
 
 
-def _serve(d, dtype, reqs, arrivals, **kw):
-    """Requests that arrive at given steps, through enqueue_requests and step; returns what each generated and why it ended."""
+def _serve(d, dtype, reqs, arrivals, poison=False, **kw):
+    """Requests that arrive at given steps, through enqueue_requests and step; returns what each generated and why it ended.
+    ``poison``: every page holds NaN before the first request, as a page may that another request has left behind."""
     from levanter_amd.config import InferenceEngineConfig
     from levanter_amd.engine import InferenceEngine, Request
 
     engine = InferenceEngine.from_pretrained(d, InferenceEngineConfig(compute_dtype=dtype, page_size=16, seed=3, **kw))
+    if poison:
+        for g in engine.cache.groups:
+            g.k_pages.fill_(float("nan"))
+            g.v_pages.fill_(float("nan"))
     seqs, pending, step = [], [Request(**r) for r in reqs], 0
     while pending or not all(s.done for s in seqs):
         while pending and arrivals[len(seqs)] <= step:
@@ -220,7 +225,7 @@ def test_random_arrivals_small_pools_and_preemption_change_no_token(trial):
     arrivals = sorted(rng.randrange(0, 40) for _ in range(n)) + [10 ** 9]
     small = dict(max_pages=rng.choice([10, 14]), max_seqs=rng.choice([3, 4, 8]), max_pages_per_seq=8, max_prefill_size=rng.choice([7, 32]))
     ahead, _ = _serve(d, dtype, reqs, arrivals, decode_lookahead=True, **small)
-    plain, _ = _serve(d, dtype, reqs, arrivals, decode_lookahead=False, **small)
+    plain, _ = _serve(d, dtype, reqs, arrivals, decode_lookahead=False, poison=True, **small)  # what a page held before is never read
     roomy, n_pre = _serve(d, dtype, reqs, [0] * n + [10 ** 9], decode_lookahead=True, max_pages=200, max_seqs=32, max_pages_per_seq=8,
                           max_prefill_size=128)
     assert n_pre == 0
