@@ -453,6 +453,9 @@ ATTN_CASES = [
     (2, 2, 128, 16, [(300, 300)], None),
     (4, 2, 64, 32, [(200, 456), (1, 30)], 300),
     (3, 1, 96, 16, [(257, 700), (130, 130)], None),
+    # eight kv heads and more: the prompt kernel sends a kv head's tiles to one XCD, here with two query heads a kv head
+    (16, 8, 64, 16, [(150, 150), (40, 200), (1, 70)], None),
+    (16, 16, 32, 16, [(130, 130)], 100),
 ]
 
 
