@@ -230,6 +230,8 @@ def serving_workload(args) -> int:
     dt = time.perf_counter() - t
     generated = sum(len(s.generated) for s in seqs)
     prompt_tokens = sum(lens)
+    slowest = max(range(len(step_ms)), key=step_ms.__getitem__)
+    print(f"[bench] {len(step_ms)} steps; the slowest was step {slowest} ({step_ms[slowest]:.1f} ms)", file=sys.stderr, flush=True)
     step_ms.sort()
     pick = lambda q: round(step_ms[min(len(step_ms) - 1, int(q * len(step_ms)))], 3)
     out = {
@@ -242,7 +244,7 @@ def serving_workload(args) -> int:
                    "global_batch": n_req, "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "prefill_chunk": chunk,
                    "page_size": ps, "max_pages": max_pages, "temperature": temperature, "parallelism": "single GPU"},
         "seconds": round(dt, 3), "generated": generated, "all_tokens_per_s": round((generated + prompt_tokens) / dt, 1),
-        "step_ms": {"p10": pick(0.1), "p50": pick(0.5), "p90": pick(0.9), "max": round(step_ms[-1], 3)},
+        "step_ms": {"p10": pick(0.1), "p50": pick(0.5), "p90": pick(0.9), "p99": pick(0.99), "max": round(step_ms[-1], 3)},
         "preemptions": engine.scheduler.n_preemptions,
     }
     print(json.dumps(out), flush=True)

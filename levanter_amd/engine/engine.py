@@ -185,8 +185,9 @@ class InferenceEngine:
 
     def warm_up(self, token_counts: Optional[Sequence[int]] = None) -> None:
         """Run prompts of several lengths once and drop them: kernels, and the GEMM library's code for the row counts
-        that prompt portions will have, are loaded before the first request is timed (a first use can take a fifth of a
-        second). ``token_counts``: tokens of each warm-up step; default: a ladder from 32 up to the largest portion."""
+        that prompt portions, decode batches and mixed steps will have, are loaded and timed before the first request is
+        (a first use can take a fifth of a second). ``token_counts``: tokens of each warm-up prompt; default: a ladder from
+        32 up to the largest portion."""
         limit = min(self.config.imputed_max_prefill_size, self.runner.max_len - 1)
         if token_counts is None:
             token_counts = [n for n in (32, 64, 128, 192, 256, 288, 320, 384, 448, 512, 640, 768, 1024, 1280, 1536, 2048) if n <= limit]
@@ -202,6 +203,18 @@ class InferenceEngine:
         most = self.config.max_seqs
         for b in sorted({b for b in (most, most // 2, 48, 32, 25) if 25 <= b <= most}):
             self.generate([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=3) for i in range(b)])
+        # a whole portion beside decoding requests: the row counts of mixed steps, which are no multiple of anything (the
+        # library keeps the kernel it timed fastest for row counts up to the same multiple of 64; timing takes a fifth of
+        # a second at 20B sizes)
+        for d in range(1, most, 64):
+            self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=4) for i in range(d)])
+            self.step()
+            self.enqueue_requests([Request(prompt_tokens=[(7 * i + 3) % v for i in range(limit)], request_id=-1 - d, max_new_tokens=1)])
+            for _ in range(8):
+                if self.scheduler.idle and self._pending is None:
+                    break
+                self.step()
+            self.reset()
         self.reset()
 
     def reset(self) -> None:
