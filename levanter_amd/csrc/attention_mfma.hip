@@ -240,8 +240,8 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
   constexpr int KCH = (64 * NCHUNK + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks of K per thread and block
   constexpr int VCH = (HD * 8 + PF_THREADS - 1) / PF_THREADS;
   static_assert(PF_THREADS % 64 == 0, "a thread's K chunks belong to one key");
-  // every thread has a chunk in every round (then staging has no branch, and the iteration below is one basic block)
-  constexpr bool K_EXACT = (64 * NCHUNK) % PF_THREADS == 0, V_EXACT = (HD * 8) % PF_THREADS == 0;
+  // Where the chunks of a block are no multiple of the threads, the threads beyond them in the last round repeat the
+  // last chunk (the same bytes to the same place): staging has no branch, and the iteration below is one basic block.
   const int ps_mask = (1 << ps_shift) - 1;
   const size_t head_elems = (size_t)HD << ps_shift;
   const size_t page_elems = (size_t)KVH * head_elems;
@@ -290,16 +290,15 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
     const int row = 4 * ((k_kk & 31) >> 3) + (k_kk & 3);
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
-      const int c = (tid >> 6) + PF_WAVES * i;
-      if (K_EXACT || c < NCHUNK) *reinterpret_cast<u32x4*>(&Ks[buf][tile][c][row][0]) = kr[i];
+      const int c = min((tid >> 6) + PF_WAVES * i, NCHUNK - 1);
+      *reinterpret_cast<u32x4*>(&Ks[buf][tile][c][row][0]) = kr[i];
     }
   };
   auto stage_v = [&](int buf, bool whole) {  // whole: the block lies in the key range, nothing to zero
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int y = tid + PF_THREADS * i;
-      if (V_EXACT || y < HD * 8)
-        *reinterpret_cast<u32x4*>(&Vs[buf][(y % (HD * 2)) >> 1][v_kk[i]]) = whole ? vr[i] : (vr[i] & first_keys_mask(vkeep[i]));
+      const int y = min(tid + PF_THREADS * i, HD * 8 - 1);
+      *reinterpret_cast<u32x4*>(&Vs[buf][(y % (HD * 2)) >> 1][v_kk[i]]) = whole ? vr[i] : (vr[i] & first_keys_mask(vkeep[i]));
     }
   };
   const int n_qt = min(PF_QT, max(0, (rows - wave_row0 + 15) / 16));  // query tiles of this wave that hold rows
