@@ -4,10 +4,11 @@
 //   tile kernel   (M > 128): a 256x256, 256x192, 256x128, 128x128 or 128x64 tile per workgroup of 4 waves, 32x32x16 MFMA,
 //                 (K split into ranges, with a second kernel for the sums, where the tiles alone would leave CUs idle)
 //                 operands staged through LDS (two buffers), the next k-tile's global loads in registers meanwhile;
-//   stream kernel (24 < M <= 128, large weights from 20 rows): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
+//   stream kernel (M <= 128; up to 24 rows where an estimate puts it ahead of the skinny kernel: long sums, workgroup counts
+//                 that do not fit the CUs): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
 //                 workgroup, the weights go straight into MFMA operand registers, K is split over workgroups
 //                 and a second kernel adds the partial sums in a fixed order;
-//   skinny kernel (M <= 24): a workgroup owns 16 output columns; its waves split K, load their part of w
+//   skinny kernel (M <= 24, see use_skinny): a workgroup owns 16 output columns; its waves split K, load their part of w
 //                 straight into MFMA operand registers (16x16x32), and their partial sums are added
 //                 through LDS in a fixed order.
 // No atomics anywhere: results are deterministic. K and lda must be multiples of 8 (16-byte operand loads);
@@ -487,22 +488,39 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 // columns x 4096 at 8 rows 28.1 -> 26.2 us, at 16 rows 33.4 -> 27.8 us; 24576 x 6144 at 16 rows 76 -> 64 us; at one
 // row and with workgroup counts that are no multiple of the CUs (18432 or 50257 columns) they lose up to 15 %.
 // Three units and 16 waves for 12288 columns x 4096: 25.1 -> 21.8 us at 16 rows, the same at 8 rows, 10 % slower at one.
+struct SkinnyShape {
+  int waves, in_flight, row_tiles, units;  // the kernel's WAVES, U, MT, NT
+};
+static SkinnyShape skinny_shape(int M, int N) {
+  const int tiles = (N + 15) / 16;
+  if (M <= 16) {
+    const bool two_units = tiles >= 1024 && (M >= 12 || (tiles / 2) % 256 == 0);
+    if (two_units) return {4, 2, 1, 2};
+    if (M >= 12 && tiles >= 720 && tiles < 1024) return {16, 1, 1, 3};  // about 256 workgroups of 48 columns
+    if (tiles >= 1024) return {4, 4, 1, 1};
+    if (tiles >= 512) return {4, 2, 1, 1};
+    return {16, 1, 1, 1};
+  }
+  // 17 .. SKINNY_MAX_M rows: two row tiles share every weight load
+  return tiles >= 512 ? SkinnyShape{4, 2, 2, 1} : SkinnyShape{16, 1, 2, 1};
+}
+
 template <typename TO>
 static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const float* bias, const float* residual, long ldr,
                           TO* out, long ldo, int M, int N, int K, int act, hipStream_t stream) {
   const int tiles = (N + 15) / 16;
-#define LEV_SKINNY(W_, U_, MT_, NT_) \
-  gemm_skinny_kernel<TO, W_, U_, 1, MT_, NT_><<<(tiles + NT_ - 1) / NT_, W_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, ldo, M, N, K, act)
-  if (M <= 16) {
-    const bool two_units = tiles >= 1024 && (M >= 12 || (tiles / 2) % 256 == 0);
-    if (two_units) LEV_SKINNY(4, 2, 1, 2);
-    else if (M >= 12 && tiles >= 720 && tiles < 1024) LEV_SKINNY(16, 1, 1, 3);  // about 256 workgroups of 48 columns
-    else if (tiles >= 1024) LEV_SKINNY(4, 4, 1, 1);
-    else if (tiles >= 512) LEV_SKINNY(4, 2, 1, 1);
-    else LEV_SKINNY(16, 1, 1, 1);
-  } else {  // 17 .. SKINNY_MAX_M rows: two row tiles share every weight load
-    if (tiles >= 512) LEV_SKINNY(4, 2, 2, 1); else LEV_SKINNY(16, 1, 2, 1);
-  }
+  const SkinnyShape sh = skinny_shape(M, N);
+#define LEV_SKINNY(W_, U_, MT_, NT_)                                                                                          \
+  if (sh.waves == W_ && sh.in_flight == U_ && sh.row_tiles == MT_ && sh.units == NT_)                                          \
+    gemm_skinny_kernel<TO, W_, U_, 1, MT_, NT_><<<(tiles + NT_ - 1) / NT_, W_ * 64, 0, stream>>>(a, lda, w, bias, residual, ldr, out, \
+                                                                                                 ldo, M, N, K, act)
+  LEV_SKINNY(4, 2, 1, 2);
+  LEV_SKINNY(16, 1, 1, 3);
+  LEV_SKINNY(4, 4, 1, 1);
+  LEV_SKINNY(4, 2, 1, 1);
+  LEV_SKINNY(16, 1, 1, 1);
+  LEV_SKINNY(4, 2, 2, 1);
+  LEV_SKINNY(16, 1, 2, 1);
 #undef LEV_SKINNY
 }
 
@@ -720,13 +738,14 @@ static int launch_splitk_reduce(const float* workspace, const float* bias, const
 struct StreamPlan {
   int waves;   // waves of a workgroup (16 columns each): 4, 8, 12 or 16
   int splits;  // k ranges
+  double cost; // the estimate, in the model's microseconds
 };
 static StreamPlan plan_stream(int M, int N, int K) {
   static const int nw[4] = {4, 8, 12, 16};
   const int chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
   const int s_max = chunks / 2 < 16 ? (chunks / 2 < 1 ? 1 : chunks / 2) : 16;  // at least two chunks each
   const double w_bytes = (double)N * K * 2.0;
-  StreamPlan best = {4, 1};
+  StreamPlan best = {4, 1, 1e30};
   double best_cost = 1e30;
   const int n_widths = w_bytes < 24e6 ? 1 : 4;  // weights of a few MB: the narrow workgroup measured best throughout
   for (int i = 0; i < n_widths; ++i) {
@@ -744,7 +763,7 @@ static StreamPlan plan_stream(int M, int N, int K) {
       if (s > 1) cost += 3.0 + 2.0 * s * M / K * (w_bytes / 4.5e6);
       if (cost < best_cost - 1e-9) {
         best_cost = cost;
-        best = {nw[i], s};
+        best = {nw[i], s, cost};
       }
     }
   }
@@ -794,13 +813,32 @@ static TilePlan plan_tiles(int M, int N, int K) {
   return best;
 }
 
-// Which kernel takes M rows: the skinny one up to 16 rows; from 17 to SKINNY_MAX_M rows (two row tiles that share the
-// weight loads) except for large weights at 20 rows and more, where the stream kernel's shared activation tile wins
-// (measured at the 7B sizes, 24 rows: 100 MB weight 30 us against 26, 134 MB 38 against 35; 33 MB 13.5 against 16).
+// Which kernel takes M <= SKINNY_MAX_M rows. The skinny kernel's time grows with the rows, because every workgroup reads all
+// of `a` (out of L2, at about 20 TB/s for all CUs together), and with workgroup counts that are no multiple of the CUs; the
+// stream kernel's hardly does, but it pays for its K ranges. An estimate of the skinny kernel in the manner of
+// plan_stream's, and a factor between the two fitted to measurements at three model sizes (microseconds, skinny / stream):
+//   4096-wide layer:  8 rows 19.5 / 24.1, 8.6 / 14.7, 24.9 / 31.6, 23.9 / 32.9 (qkv, proj, fc, second MLP matrix);
+//                     24 rows 27.8 / 25.2, 12.6 / 15.9, 35.8 / 33.2, 35.3 / 33.6
+//   6144-wide layer:  8 rows 48.3 / 53.7, 20.6 / 21.4, 55.2 / 59.2, 67.0 / 60.3; 16 rows 55.3 / 54.5, 25.0 / 22.0, 60.3 / 60.3,
+//                     86.1 / 60.6 (384 workgroups of the skinny kernel: one and a half rounds); 24 rows 66 / 55, 32 / 23, 80 / 62, 104 / 62
+//   1600-wide layer:  8 rows 7.0 / 8.1, 4.7 / 7.1, 8.3 / 9.5, 10.8 / 10.8; 16 rows 7.3 / 8.2, 4.8 / 7.2, 9.0 / 10.0, 13.6 / 11.0
+//   heads (50257 columns) of 4096 / 6144 / 1600 / 768: 8 rows 81 / 87, 125 / 152, 34.6 / 34.3, 17.0 / 20.6; 24 rows 108 / 91, 169 / 156,
+//                     46.5 / 35.9, 24.3 / 22.2
+// Over the 112 cases measured (1 to 24 rows) the choice made here is on average 1 % behind the better kernel; the rule before
+// it (rows alone, with one exception for large weights) 4 %, and up to 70 % on the long sums of the 6144-wide layer.
+static double skinny_estimate(int M, int N, int K) {
+  const SkinnyShape sh = skinny_shape(M, N);
+  const long wgs = ((N + 15) / 16 + sh.units - 1) / sh.units;
+  const long r = (wgs + 255) / 256;  // workgroups of the slowest CU
+  const double w_bytes = (double)N * K * 2.0, a_bytes = (double)wgs * M * K * 2.0;
+  const double t = w_bytes / 7.5e6 + a_bytes / 20e6;
+  double cost = 3.0 + t * (wgs >= 256 ? (double)r * 256.0 / wgs : 256.0 / wgs);
+  if (sh.row_tiles == 2) cost *= 1.2;
+  return cost;
+}
 static bool use_skinny(int M, int N, int K) {
-  if (M <= 16) return true;
   if (M > SKINNY_MAX_M) return false;
-  return !(M >= 20 && (double)N * K * 2.0 >= 64e6);
+  return skinny_estimate(M, N, K) <= 1.3 * plan_stream(M, N, K).cost;
 }
 
 // Into how many ranges the sum over K is split (1: the kernel finishes its outputs itself).

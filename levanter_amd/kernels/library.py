@@ -326,11 +326,12 @@ class HipKernels:
         (K >= 4 N) below 1,024 rows and weights of a few MB below 320 rows. From 25 to 255 rows: wide outputs of large
         weights (N >= 2 K, 32 MB and more: 7B qkv and fc at 64 rows 28.1 / 25.3 and 37.1 / 33.5 us, ours with the kernel that
         adds its K ranges; at 160 rows 49.7 / 37.2 and 55.7 / 41.6); ours keep N = K (17.4 / 16.3 at 64 rows, 22.1 / 24.6 at
-        128) and K = 4 N (36.8 / 41.2, 43.5 / 81.1)."""
+        128) and K = 4 N (36.8 / 41.2, 43.5 / 81.1), and below 96 rows the largest weights (more than 256 MB: the fc of a
+        6144-wide layer 64.4 / 72.4 at 32 rows, 70.1 / 75.4 at 64, 85.0 / 84.4 at 128; its qkv, 216 MB, 58.9 / 57.6 and 62.3 / 59.7)."""
         if act not in cls.LIBRARY_ACTIVATIONS or M < cls.LIBRARY_MIN_ROWS:
             return False
         if M < 256:
-            return N >= 2 * K and N * K >= (1 << 24)
+            return N >= 2 * K and N * K >= (1 << 24) and not (M < 96 and N * K > (1 << 27))
         if M < 320 and N * K < (1 << 24):
             return False
         return not (K >= 4 * N and M < 1024)

@@ -361,6 +361,19 @@ def test_the_vendor_library_s_product_inside_a_recorded_graph(K, M, K_, N, act, 
         assert bool(out.float().abs().sum() > 0)
 
 
+def test_which_kernel_takes_a_few_rows(K):
+    """Up to 24 rows an estimate decides between the kernel whose workgroups each read all of the activations (fast while
+    they are few and the workgroups fit the CUs) and the one that shares them and splits the sum over K (ranges > 1): the
+    decode batches of the 4096-wide layer stay where they were measured best, long sums and awkward widths move early."""
+    ranges = K._unit("gemm_mfma").lev_linear_mfma_ranges
+    for M in (1, 8, 16):
+        assert all(ranges(M, N, K_) == 1 for N, K_ in [(12288, 4096), (4096, 4096), (16384, 4096), (4096, 16384), (50257, 4096)]), M
+    assert ranges(24, 12288, 4096) > 1 and ranges(24, 16384, 4096) > 1 and ranges(24, 4096, 4096) == 1
+    assert ranges(8, 6144, 24576) > 1 and ranges(16, 6144, 24576) > 1  # 384 workgroups: one and a half rounds of the CUs
+    assert ranges(4, 18432, 6144) == 1 and ranges(24, 18432, 6144) > 1
+    assert ranges(8, 1600, 1600) == 1 and ranges(16, 1600, 6400) > 1
+
+
 def test_which_products_go_to_the_vendor_library(K):
     none, gelu, silu = 0, 1, 4
     assert not K.use_library(24, 12288, 4096, none) and K.use_library(25, 12288, 4096, none) and K.use_library(256, 12288, 4096, none)
@@ -368,6 +381,7 @@ def test_which_products_go_to_the_vendor_library(K):
     assert K.use_library(2048, 16384, 4096, gelu) and not K.use_library(2048, 16384, 4096, silu)
     assert not K.use_library(512, 4096, 16384, none) and K.use_library(1024, 4096, 16384, none)  # long sums into a narrow output
     assert not K.use_library(256, 4800, 1600, none) and K.use_library(320, 4800, 1600, none)  # small weights
+    assert K.use_library(32, 18432, 6144, none) and not K.use_library(32, 24576, 6144, gelu) and K.use_library(128, 24576, 6144, gelu)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
