@@ -219,6 +219,7 @@ def serving_workload(args) -> int:
     engine.reset()
     engine.warm_up()
     step_ms = []
+    print("[bench] warm-up done, the timed run starts", file=sys.stderr, flush=True)
     seqs = engine.enqueue_requests(requests(2))
     torch.cuda.synchronize()
     t = time.perf_counter()

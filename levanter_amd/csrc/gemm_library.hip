@@ -6,7 +6,8 @@
 // Everything else (other activations, shapes it has no kernel for) returns LEV_LIBRARY_UNSUPPORTED and the caller
 // runs the hand-written kernel. Which of the library's kernels runs a shape is not left to its heuristic alone: for
 // 256 rows and more the heuristic's candidates are timed once (its first choice is up to twice slower than its best on row
-// counts that are no multiple of the tile, 2,052 rows for instance) and row counts of one bucket of 64 share the result. In the library's column-major terms the row-major problem is
+// counts that are no multiple of the tile, 2,052 rows for instance); the other row counts up to the same multiple of 64 try
+// only that kernel against the heuristic's first. In the library's column-major terms the row-major problem is
 //   D^T [N x M] = w_cm^T [N x K] . a_cm [K x M]  (+ C^T),  with w_cm = w seen as K x N (ld K), a_cm = a seen as K x M (ld lda),
 // so that the bias, one value per row of D^T, is the per-output-column bias of the row-major result.
 #include <hipblaslt/hipblaslt.h>
@@ -124,14 +125,14 @@ int tune_level() {
   return level;
 }
 
-// Times every candidate of a plan on the call's own operands, writing to a buffer of its own (a product into the residual
-// stream adds to its output, so the real output cannot take repeated runs), and keeps the fastest. The heuristic's order is
-// a table look-up by size; on this chip its first kernel is often not the fastest one for the shape at hand.
-// Allocates and synchronises: called only outside a stream capture, once per shape and process.
-int time_candidates(hipblasLtHandle_t handle, Plan* p, const void* a, const void* w, const float* residual, void* workspace, int M,
-                     int N, long ldo, int out_dtype, hipStream_t stream) {
+// Times the given kernels on the call's own operands, writing to a buffer of its own (a product into the residual stream
+// adds to its output, so the real output cannot take repeated runs), and gives the plan the fastest. The heuristic's order
+// is a table look-up by size; on this chip its first kernel is often not the fastest one for the shape at hand.
+// Allocates and synchronises: called only outside a stream capture. Returns the library's index of the kernel kept, or -1.
+int time_candidates(hipblasLtHandle_t handle, Plan* p, const std::vector<hipblasLtMatmulHeuristicResult_t>& candidates, const void* a,
+                    const void* w, const float* residual, void* workspace, int M, int N, long ldo, int out_dtype, hipStream_t stream) {
   p->timed = true;
-  if (p->candidates.size() < 2) return -1;
+  if (candidates.size() < 2) return -1;
   auto t_begin = std::chrono::steady_clock::now();
   const size_t bytes = (size_t)M * (size_t)ldo * (out_dtype == LEV_F32 ? 4 : 2);
   void* scratch = nullptr;
@@ -147,8 +148,8 @@ int time_candidates(hipblasLtHandle_t handle, Plan* p, const void* a, const void
   const void* c = residual ? (const void*)residual : (const void*)scratch;
   float best = -1.0f;
   int best_i = 0;
-  for (size_t i = 0; i < p->candidates.size(); ++i) {
-    const hipblasLtMatmulHeuristicResult_t& cand = p->candidates[i];
+  for (size_t i = 0; i < candidates.size(); ++i) {
+    const hipblasLtMatmulHeuristicResult_t& cand = candidates[i];
     bool ok = true;
     float ms = 0.0f;
     for (int run = 0; run <= LEV_LIB_TUNE_RUNS && ok; ++run) {  // run 0 loads the kernel and is not timed
@@ -167,8 +168,8 @@ int time_candidates(hipblasLtHandle_t handle, Plan* p, const void* a, const void
     if (best < 0.0f || ms < best) { best = ms; best_i = (int)i; }
   }
   if (best >= 0.0f) {
-    p->algo = p->candidates[best_i].algo;
-    p->workspace = p->candidates[best_i].workspaceSize;
+    p->algo = candidates[best_i].algo;
+    p->workspace = candidates[best_i].workspaceSize;
     if (tune_level() >= 2)
       fprintf(stderr, "linear (library) M=%d N=%d: kept candidate %d after %.1f ms\n", M, N, best_i,
               std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t_begin).count());
@@ -180,19 +181,14 @@ int time_candidates(hipblasLtHandle_t handle, Plan* p, const void* a, const void
   return best >= 0.0f ? hipblaslt_ext::getIndexFromAlgo(p->algo) : -1;
 }
 
-// Gives a plan the kernel that timing chose for another row count of its bucket, if that kernel takes this problem too.
-bool adopt_index(hipblasLtHandle_t handle, Plan* p, int index, bool residual, size_t max_workspace) {
-  std::vector<int> indices(1, index);
-  std::vector<hipblasLtMatmulHeuristicResult_t> found;
-  if (hipblaslt_ext::getAlgosFromIndex(handle, indices, found) != HIPBLAS_STATUS_SUCCESS || found.empty()) return false;
-  const float alpha = 1.0f, beta = residual ? 1.0f : 0.0f;
-  size_t need = 0;
-  if (hipblaslt_ext::matmulIsAlgoSupported(handle, p->desc, &alpha, p->lw, p->la, &beta, p->lc, p->ld, found[0].algo, need) !=
-          HIPBLAS_STATUS_SUCCESS || need > max_workspace)
-    return false;
-  p->algo = found[0].algo;
-  p->workspace = need;
-  return true;
+// The kernel that timing chose for another row count of the plan's bucket, if the heuristic offers it for this row count
+// too. (Asking the library for a kernel by its index instead makes it load its whole catalogue: a second at its first use.)
+const hipblasLtMatmulHeuristicResult_t* candidate_of_index(const Plan* p, int index) {
+  for (const hipblasLtMatmulHeuristicResult_t& cand : p->candidates) {
+    hipblasLtMatmulAlgo_t algo = cand.algo;
+    if (hipblaslt_ext::getIndexFromAlgo(algo) == index) return &cand;
+  }
+  return nullptr;
 }
 
 }  // namespace
@@ -232,19 +228,31 @@ extern "C" int lev_linear_library(const void* a, long lda, const void* w, const 
     LIB_CHECK(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp)));
   }
   if (!plan.timed && M >= LEV_LIB_TUNE_MIN_ROWS && tune_level() >= 1) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) { (void)hipGetLastError(); capturing = hipStreamCaptureStatusActive; }
+    const bool may_time = capturing == hipStreamCaptureStatusNone;
     const PlanKey bucket(dev, rows_bucket(M), N, K, lda, residual ? ldr : 0, ldo, (int)epilogue, out_dtype, residual ? 1 : 0);
     auto known = g_timed_index.find(bucket);
-    if (known != g_timed_index.end()) {
-      plan.timed = true;  // whether it fits or not: the plan is settled
-      const bool fits = known->second >= 0 && adopt_index(handle, &plan, known->second, residual != nullptr, (size_t)workspace_bytes);
-      if (tune_level() >= 2)
-        fprintf(stderr, "linear (library) M=%d N=%d K=%d: kernel %d of its bucket %s\n", M, N, K, known->second,
-                fits ? "taken" : "does not fit");
+    if (known == g_timed_index.end()) {
+      if (may_time)
+        g_timed_index[bucket] = time_candidates(handle, &plan, plan.candidates, a, w, residual, workspace, M, N, ldo, out_dtype, stream);
     } else {
-      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-      if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) { (void)hipGetLastError(); capturing = hipStreamCaptureStatusActive; }
-      if (capturing == hipStreamCaptureStatusNone)
-        g_timed_index[bucket] = time_candidates(handle, &plan, a, w, residual, workspace, M, N, ldo, out_dtype, stream);
+      // Another row count of the bucket has been timed: its kernel against the heuristic's first for this row count (a
+      // kernel that won at 264 rows can lose at 320, where its tiles divide the rows differently), not all sixteen again.
+      plan.timed = true;  // whether the bucket's kernel is on offer or not: the plan is settled
+      const hipblasLtMatmulHeuristicResult_t* theirs = known->second >= 0 ? candidate_of_index(&plan, known->second) : nullptr;
+      if (tune_level() >= 2)
+        fprintf(stderr, "linear (library) M=%d N=%d K=%d: kernel %d of its bucket is %s\n", M, N, K, known->second,
+                theirs == &plan.candidates[0] ? "the heuristic's first" : (theirs ? "on offer" : "not on offer"));
+      if (theirs && theirs != &plan.candidates[0]) {
+        if (may_time) {
+          std::vector<hipblasLtMatmulHeuristicResult_t> two = {*theirs, plan.candidates[0]};
+          time_candidates(handle, &plan, two, a, w, residual, workspace, M, N, ldo, out_dtype, stream);
+        } else {
+          plan.algo = theirs->algo;
+          plan.workspace = theirs->workspaceSize;
+        }
+      }
     }
   }
   if (plan.workspace > 0 && !workspace)

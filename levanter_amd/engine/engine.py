@@ -206,11 +206,12 @@ class InferenceEngine:
         # a whole portion beside decoding requests: the row counts of mixed steps, which are no multiple of anything (the
         # library keeps the kernel it timed fastest for row counts up to the same multiple of 64; timing takes a fifth of
         # a second at 20B sizes)
+        rounds = self.config.max_rounds  # decode steps that may pass before a waiting request is admitted
         for d in range(1, most, 64):
-            self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=4) for i in range(d)])
+            self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=rounds + 4) for i in range(d)])
             self.step()
             self.enqueue_requests([Request(prompt_tokens=[(7 * i + 3) % v for i in range(limit)], request_id=-1 - d, max_new_tokens=1)])
-            for _ in range(8):
+            for _ in range(rounds + 8):
                 if self.scheduler.idle and self._pending is None:
                     break
                 self.step()

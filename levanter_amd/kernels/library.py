@@ -323,7 +323,9 @@ class HipKernels:
     def use_library(cls, M: int, N: int, K: int, act: int) -> bool:
         """Which products go to the vendor library: those with an epilogue it has, at the shapes where it was measured
         ahead on MI355X (widths of GPT-2 7B and XL, with epilogues). From 256 rows: all but long sums into narrow outputs
-        (K >= 4 N) below 1,024 rows and weights of a few MB below 320 rows. From 25 to 255 rows: wide outputs of large
+        (K >= 4 N) below 1,024 rows and, below 320 rows, weights of a few MB unless the output is wide (a 1600-wide layer at 264
+        rows, ours / library with its kernel timed: qkv 18.3 / 16.7, fc 24.8 / 18.8, proj 11.9 / 14.2, second MLP matrix 22.7 / 20.4 but
+        20.1 / 23.5 at 256 and 22.9 / 23.5 at 288). From 25 to 255 rows: wide outputs of large
         weights (N >= 2 K, 32 MB and more: 7B qkv and fc at 64 rows 28.1 / 25.3 and 37.1 / 33.5 us, ours with the kernel that
         adds its K ranges; at 160 rows 49.7 / 37.2 and 55.7 / 41.6); ours keep N = K (17.4 / 16.3 at 64 rows, 22.1 / 24.6 at
         128) and K = 4 N (36.8 / 41.2, 43.5 / 81.1), and below 96 rows the largest weights (more than 256 MB: the fc of a
@@ -333,7 +335,7 @@ class HipKernels:
         if M < 256:
             return N >= 2 * K and N * K >= (1 << 24) and not (M < 96 and N * K > (1 << 27))
         if M < 320 and N * K < (1 << 24):
-            return False
+            return N >= 2 * K
         return not (K >= 4 * N and M < 1024)
 
     # ---- cache write -----------------------------------------------------------------------

@@ -315,3 +315,13 @@ def test_max_rounds_is_the_number_of_decode_steps_between_two_looks_at_the_queue
     assert late[0].generated == [52, 53, 54]
     engine.reset()
     assert all_released(engine)
+
+
+def test_warm_up_meets_the_row_counts_of_serving():
+    """Prompts up to a whole portion alone, batches of single tokens, and a whole portion beside decoding requests (their
+    number of rows is what the matrix products of a mixed step see); afterwards the engine is as it was."""
+    engine, model = make_engine(max_pages=4096, max_seqs=64, max_pages_per_seq=64, max_prefill_size=256, max_seqs_in_prefill=64)
+    engine.warm_up(token_counts=[32, 256])
+    shapes = {(len(b), sum(b)) for b in model.batches}
+    assert {(1, 32), (1, 256), (64, 64), (32, 32), (2, 257)} <= shapes, sorted(shapes)
+    assert engine.scheduler.idle and all_released(engine)
