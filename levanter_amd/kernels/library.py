@@ -333,7 +333,11 @@ class HipKernels:
         if act not in cls.LIBRARY_ACTIVATIONS or M < cls.LIBRARY_MIN_ROWS:
             return False
         if M < 256:
-            return N >= 2 * K and N * K >= (1 << 24) and not (M < 96 and N * K > (1 << 27))
+            if N < 2 * K:
+                return False
+            if N * K < (1 << 24):
+                return M >= 128  # a 1600-wide layer: qkv 16.5 / 14.2 at 128 rows, 17.3 / 14.5 at 192, but 12.8 / 14.3 at 64
+            return not (M < 96 and N * K > (1 << 27))
         if M < 320 and N * K < (1 << 24):
             return N >= 2 * K
         return not (K >= 4 * N and M < 1024)

@@ -381,6 +381,7 @@ def test_which_products_go_to_the_vendor_library(K):
     assert K.use_library(2048, 16384, 4096, gelu) and not K.use_library(2048, 16384, 4096, silu)
     assert not K.use_library(512, 4096, 16384, none) and K.use_library(1024, 4096, 16384, none)  # long sums into a narrow output
     assert K.use_library(256, 4800, 1600, none) and not K.use_library(256, 1600, 1600, none) and K.use_library(320, 1600, 1600, none)  # small weights
+    assert not K.use_library(64, 4800, 1600, none) and K.use_library(128, 4800, 1600, none) and not K.use_library(128, 1600, 1600, none)
     assert K.use_library(32, 18432, 6144, none) and not K.use_library(32, 24576, 6144, gelu) and K.use_library(128, 24576, 6144, gelu)
 
 
