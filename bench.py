@@ -31,6 +31,15 @@ def load_baseline_config():
             "n_positions": 2048, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
 
 
+# the other sizes of the reference's configurations (config/gpt2_xl.yaml, config/gpt2_20b.yaml), for --shape
+OTHER_SHAPES = {
+    "xl": {"model_type": "gpt2", "n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400, "vocab_size": 50257,
+           "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"},
+    "20b": {"model_type": "gpt2", "n_layer": 44, "n_embd": 6144, "n_head": 64, "n_inner": 24576, "vocab_size": 50257,
+            "n_positions": 2048, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"},
+}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -42,6 +51,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
+    ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
+                    help="layer sizes of the decode workload: 7b is the contract's; xl and 20b measure the same step at the other "
+                         "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
     ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b"],
                     help="decode: the contract above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
                          "through InferenceEngine.generate; they print their own line")
@@ -58,7 +70,8 @@ def main() -> int:
     if args.workload != "decode":
         return serving_workload(args)
 
-    raw = load_baseline_config()
+    raw = load_baseline_config() if args.shape == "7b" else dict(OTHER_SHAPES[args.shape])
+    shape_name = {"7b": "GPT-2 7B", "xl": "GPT-2 XL", "20b": "GPT-2 20B"}[args.shape]
     full_layers = raw["n_layer"]
     if args.layers is not None:
         raw["n_layer"] = args.layers
@@ -143,11 +156,12 @@ def main() -> int:
     step_bytes = weight_bytes + args.batch * ctx_mean * kv_bytes_per_token
     achieved = step_bytes / (dt / args.steps) / 1e9
     out = {
-        "metric": "decode tok/s @ batch 8, GPT-2 7B shape, bf16" if args.batch == 8 else f"decode tok/s @ batch {args.batch}, GPT-2 7B shape",
+        "metric": (f"decode tok/s @ batch 8, {shape_name} shape, bf16" if args.batch == 8 and args.dtype == "bfloat16"
+                   else f"decode tok/s @ batch {args.batch}, {shape_name} shape"),
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
-        "config": {"model": "gpt2_7b shape", "n_layer": L, "n_layer_full": full_layers, "n_embd": D, "n_head": cfg.n_head,
+        "config": {"model": f"gpt2_{args.shape} shape", "n_layer": L, "n_layer_full": full_layers, "n_embd": D, "n_head": cfg.n_head,
                    "head_dim": cfg.head_dim, "n_inner": F, "vocab_size": V, "n_positions": cfg.n_positions,
                    "global_batch": args.batch, "seq_len": args.prompt_len + GENERATED, "prompt_len": args.prompt_len,
                    "generated": GENERATED, "ctx_mean": round(ctx_mean, 1), "page_size": ps, "parallelism": "single GPU"},
