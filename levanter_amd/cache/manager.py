@@ -15,7 +15,7 @@ runs; fixed-size state lives in ``StateSlots`` indexed by the request's slot.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np

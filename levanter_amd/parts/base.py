@@ -10,7 +10,7 @@ compute dtype ``h``; mixers and feed-forwards add their result to ``x`` in place
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, Optional
 
 import torch
 
