@@ -51,6 +51,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
+    ap.add_argument("--prefill-len", type=int, default=2048, help="with --prefill-only: tokens of the prompt (the contract's point is 2,048)")
     ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
                     help="layer sizes of the decode workload: 7b is the contract's; xl and 20b measure the same step at the other "
                          "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
@@ -147,7 +148,10 @@ def main() -> int:
         return {"value": round(T / best, 1), "tokens": T, "ms": round(best * 1e3, 3), "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
 
     if args.prefill_only:
-        print(json.dumps({"prefill": prefill_run(2048, 4)}), flush=True)
+        if not 1 <= args.prefill_len < cfg.n_positions + 1:
+            print(f"bench.py: --prefill-len {args.prefill_len} does not fit n_positions {cfg.n_positions}")
+            return 2
+        print(json.dumps({"prefill": prefill_run(args.prefill_len, 4), "model": f"gpt2_{args.shape} shape"}), flush=True)
         return 0
 
     dt, ctx_mean = decode_run(args.batch, args.steps, args.warmup, seed=1)
