@@ -135,7 +135,8 @@ class InferenceEngine:
         finished = self.scheduler.commit(pend.plan, toks, lps)
         if nxt is not None:
             if all(e.seq.done for e in nxt.plan):  # every request of the step launched ahead has ended meanwhile
-                self.sampler.read(nxt.sample)
+                if nxt.sample is not None:
+                    self.sampler.read(nxt.sample)
             else:
                 self._pending = nxt
         return finished
