@@ -48,8 +48,6 @@ class InferenceEngineConfig:
     """Seed from which per-request sampling keys are derived (engine.py:100)."""
     enable_logprobs: bool = False
     """Return the log-probability of every generated token (engine.py:102)."""
-    max_state_slots: Optional[int] = None
-    """Slots of fixed-size per-request state; None: max_seqs. (Ours.)"""
     decode_lookahead: bool = True
     """Launch the next step of single tokens before the tokens of the running one are read back. (Ours.)"""
 

@@ -33,6 +33,9 @@ class Gpt2Config(LmConfig):
     initializer_range: float = 0.02
     tie_word_embeddings: bool = True
     use_bias: bool = True  # the reference's own flag (gpt2.py:57); absent from config.json means True
+    scale_attn_weights: bool = True
+    """A key of GPT-2's config.json that the reference does not read (gpt2.py:102-117): scores are always scaled by
+    1/sqrt(head size) (src/levanter/layers/attention.py:153-154). ``false`` is refused rather than ignored."""
     attn_pdrop: float = 0.0
     embd_pdrop: float = 0.0
     resid_pdrop: float = 0.0
@@ -52,6 +55,8 @@ class Gpt2Config(LmConfig):
             )
         if not self.layer_norm_epsilon > 0:
             raise ConfigError(f"gpt2: layer_norm_epsilon must be positive, got {self.layer_norm_epsilon!r}")
+        if not self.scale_attn_weights:
+            raise ConfigError("gpt2: scale_attn_weights=false is not supported (scores are always scaled by 1/sqrt(head size))")
         if not self.tie_word_embeddings:
             # the reference has no untied path: the head is the token table (gpt2.py:361-362)
             raise ConfigError("gpt2: tie_word_embeddings=false is not supported (the head is the token table)")

@@ -68,7 +68,9 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, floa
 // partial != null: the row is first brought up to date. A matrix product that split its sum into S ranges has left
 // them in partial [S][M][D] instead of adding them to x (its residual); here x[row] += (partial[0] + .. + partial[S-1]
 // + lin_bias), in that order, is stored back and normalised in the same pass: one kernel where a reduction kernel and a
-// norm kernel would each read and write the row.
+// norm kernel would each read and write the row. With a selection of rows (rows != null) nothing is stored back: the rows
+// that are left out stay unfinished anyway, so x as a whole is of no use afterwards, and a row that the selection names
+// twice would otherwise be read by one workgroup while another has already stored its new value.
 template <typename TO, int NT, int NV>
 __global__ void __launch_bounds__(NT)
 norm_reg_kernel(float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b, TO* __restrict__ out,
@@ -114,7 +116,7 @@ norm_reg_kernel(float* __restrict__ x, const float* __restrict__ w, const float*
           t.x += lb.x; t.y += lb.y; t.z += lb.z; t.w += lb.w;
         }
         v[i].x = t.x + v[i].x; v[i].y = t.y + v[i].y; v[i].z = t.z + v[i].z; v[i].w = t.w + v[i].w;
-        *reinterpret_cast<float4*>(xr + d) = v[i];
+        if (!rows) *reinterpret_cast<float4*>(xr + d) = v[i];
       }
     }
   }
@@ -214,9 +216,10 @@ extern "C" int lev_norm(const float* x, const float* w, const float* b, void* ou
   return lev_check_launch("norm");
 }
 
-// The norm of rows that a matrix product has not finished yet: x [M][D] += partial[0] + .. + partial[S-1] + lin_bias for the
-// rows that are normalised (all M, or rows[0 .. n_rows)), stored back, then the norm as in lev_norm. Returns 1, with
-// nothing launched, if this width or alignment has no such kernel.
+// The norm of rows that a matrix product has not finished yet: x [M][D] + partial[0] + .. + partial[S-1] + lin_bias, then the
+// norm as in lev_norm. rows == null: all M rows, and the sums are stored back into x, which is then finished. rows given:
+// only those rows are summed and normalised and x is left as it was (unfinished; a row may be named more than once).
+// Returns 1, with nothing launched, if this width or alignment has no such kernel.
 extern "C" int lev_norm_pending(float* x, const float* partial, int S, const float* lin_bias, const float* w, const float* b,
                                 void* out, const int* rows, int n_rows, int M, int D, float eps, int rms, int out_dtype,
                                 hipStream_t stream) {
@@ -364,8 +367,10 @@ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
   out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
+// u = (top 23 bits + 1/2) / 2^23: every value is a float32 exactly (24 significant bits at most), the smallest is 2^-24 and the
+// largest 1 - 2^-24, so both logarithms are finite. (With 24 bits the largest sum would round up to 1 and the noise to +inf.)
 __device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
-  const float u = ((float)(bits >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+  const float u = ((float)(bits >> 9) + 0.5f) * (1.0f / 8388608.0f);
   return -logf(-logf(u));
 }
 

@@ -44,7 +44,7 @@ class InferenceEngine:
         self.runner = ModelRunner(model, self.cache, env, allocate=allocate)
         self.sampler = Sampler(env.kernels, env.device)
         self.scheduler = Scheduler(self.cache, config, self.runner.max_len)
-        self.stats = {"steps": 0, "commits": 0, "tokens_in": 0, "device_s": 0.0}
+        self.stats = {"steps": 0, "commits": 0, "tokens_in": 0, "launch_s": 0.0}
         self._pending: Optional[_Launched] = None  # a step launched ahead of the one being committed
 
     # ---- construction -------------------------------------------------------------------------
@@ -161,7 +161,7 @@ class InferenceEngine:
             sample = self.sampler.launch(logits, temps, keys, positions)
         self.stats["steps"] += 1
         self.stats["tokens_in"] += sum(len(e.tokens) for e in plan)
-        self.stats["device_s"] += time.perf_counter() - t0
+        self.stats["launch_s"] += time.perf_counter() - t0  # the host's time to plan the tables and launch the kernels
         return _Launched(plan, sample)
 
     def generate(self, requests: Sequence[Request]) -> GenerationResult:
@@ -187,31 +187,45 @@ class InferenceEngine:
     def warm_up(self, token_counts: Optional[Sequence[int]] = None) -> None:
         """Run prompts of several lengths once and drop them: kernels, and the GEMM library's code for the row counts
         that prompt portions, decode batches and mixed steps will have, are loaded and timed before the first request is
-        (a first use can take a fifth of a second). ``token_counts``: tokens of each warm-up prompt; default: a ladder from
-        32 up to the largest portion."""
-        limit = min(self.config.imputed_max_prefill_size, self.runner.max_len - 1)
+        (a first use can take a fifth of a second). ``token_counts``: prompt tokens of each warm-up step; default: a ladder
+        from 32 up to ``max_prefill_size``. A step may hold more prompt tokens than one request can (the budget is the
+        step's, the length limit the request's): such a count is made of several requests that are admitted together."""
+        one = self.runner.max_len - 1  # the longest prompt that still generates a token
+        budget = self.config.imputed_max_prefill_size
+        most = self.config.max_seqs
+        limit = min(budget, one * min(most, self.config.max_seqs_in_prefill))
         if token_counts is None:
             token_counts = [n for n in (32, 64, 128, 192, 256, 288, 320, 384, 448, 512, 640, 768, 1024, 1280, 1536, 2048) if n <= limit]
-            if limit not in token_counts:
-                token_counts.append(limit)
+            for n in (min(budget, one), limit):
+                if n not in token_counts:
+                    token_counts.append(n)
         if not self.scheduler.idle or self._pending is not None:
             raise RuntimeError("warm_up() runs on an idle engine")
         v = self.model.vocab_size
+
+        def prompts(n: int, first_id: int) -> List[Request]:
+            """Requests whose prompts have n tokens together, each as long as a request may be but the last."""
+            out = []
+            while n > 0:
+                k = min(n, one)
+                out.append(Request(prompt_tokens=[(7 * i + 3) % v for i in range(k)], request_id=first_id - len(out), max_new_tokens=1))
+                n -= k
+            return out
+
         for n in token_counts:
-            n = max(1, min(int(n), limit))
-            self.generate([Request(prompt_tokens=[(7 * i + 3) % v for i in range(n)], request_id=-1, max_new_tokens=1)])
+            self.generate(prompts(max(1, min(int(n), limit)), -1))
+            self.reset()
         # batches of decoding requests: the head and the products of a decode step at the row counts where the library takes them
-        most = self.config.max_seqs
         for b in sorted({b for b in (most, most // 2, 48, 32, 25) if 25 <= b <= most}):
             self.generate([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=3) for i in range(b)])
-        # a whole portion beside decoding requests: the row counts of mixed steps, which are no multiple of anything (the
-        # library keeps the kernel it timed fastest for row counts up to the same multiple of 64; timing takes a fifth of
-        # a second at 20B sizes)
+        # a whole step's worth of prompt tokens beside decoding requests: the row counts of mixed steps, which are no multiple
+        # of anything (the library keeps the kernel it timed fastest for row counts up to the same multiple of 64; timing
+        # takes a fifth of a second at 20B sizes)
         rounds = self.config.max_rounds  # decode steps that may pass before a waiting request is admitted
         for d in range(1, most, 64):
             self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=rounds + 4) for i in range(d)])
             self.step()
-            self.enqueue_requests([Request(prompt_tokens=[(7 * i + 3) % v for i in range(limit)], request_id=-1 - d, max_new_tokens=1)])
+            self.enqueue_requests(prompts(min(limit, one * max(1, min(most - d, self.config.max_seqs_in_prefill))), -1 - d))
             for _ in range(rounds + 8):
                 if self.scheduler.idle and self._pending is None:
                     break

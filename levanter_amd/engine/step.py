@@ -137,7 +137,7 @@ class ModelRunner:
         ``pad_batch`` (steps of single tokens that may be replayed as a graph): the batch is filled up to
         ``graph_batch_bucket`` tokens with ghosts, so that a serving run whose requests end one by one meets a
         handful of shapes instead of one per batch size. A ghost is a token 0 at position 0 that reads the first
-        request's first key, is written nowhere (destination -1) and whose logits nobody reads."""
+        request's first key, is written nowhere (destination -1) and whose logits (of its own row) nobody reads."""
         cache, ps = self.cache, self.cache.page_size
         S = len(entries)
         T = sum(len(e.tokens) for e in entries)
@@ -177,7 +177,7 @@ class ModelRunner:
                 token_seq = np.concatenate([token_seq, np.zeros(ghosts, np.int32)])
                 seq_slots = np.concatenate([seq_slots, np.full(ghosts, seq_slots[0], np.int32)])
                 decode.extend(range(T, T + ghosts))
-                rows.extend([rows[0]] * ghosts)
+                rows.extend(range(T, T + ghosts))  # a ghost's logits are its own row's: no row is wanted twice
                 S += ghosts
                 T += ghosts
         # the attention kernel pairs tile i with tile n - 1 - i: sorted by falling key range, pairs have equal work

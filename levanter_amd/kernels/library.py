@@ -203,7 +203,9 @@ class HipKernels:
     def norm(self, x, weight, bias, eps: float, out, rows=None, rms: bool = False, pending: Optional[PendingSum] = None) -> None:
         """LayerNorm (or RMSNorm) of float32 rows into ``out`` (compute dtype). rows: int32 row indices into x.
         ``pending``: an unfinished product into ``x`` (see ``PendingSum``); its ranges are added to the rows that are
-        normalised, stored back into ``x`` and normalised in one kernel."""
+        normalised and normalised in one kernel. Without ``rows`` the sums are stored back and ``x`` is finished; with
+        ``rows`` (which may name a row twice) only the selection is computed and ``x`` must not be read again: it is
+        either left unfinished or finished, depending on whether the width has a fused kernel."""
         _dev(x, weight, bias, out, rows)
         D = x.shape[1]
         n = out.shape[0]

@@ -37,8 +37,10 @@ class CausalSelfAttention(Mixer):
         self.window = p.get("window")
         if self.n_heads % self.n_kv_heads != 0:
             raise ValueError(f"attention: {self.n_heads} heads are not a multiple of {self.n_kv_heads} key/value heads")
-        if self.head_dim % 16 != 0:
-            raise ValueError(f"attention: head_dim={self.head_dim} must be a multiple of 16")
+        # the cache keeps keys in chunks of 8 head dimensions; the matrix-core kernels need multiples of 16
+        step = 16 if env.dtype == torch.bfloat16 else 8
+        if self.head_dim % step != 0:
+            raise ValueError(f"attention: head_dim={self.head_dim} must be a multiple of {step} in {env.dtype}")
         layout = p.get("weight_layout", "out_in")
         self.qkv = Linear(tensors["qkv.weight"], tensors.get("qkv.bias"), layout, env)
         self.out = Linear(tensors["out.weight"], tensors.get("out.bias"), layout, env)

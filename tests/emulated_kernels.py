@@ -47,6 +47,16 @@ def philox4x32_10(c0, c1, c2, c3, k0, k1):
     return c0, c1, c2, c3
 
 
+def uniform_from_bits(bits: np.ndarray) -> np.ndarray:
+    """(top 23 bits + 1/2) / 2^23 in float32: exact, inside (0, 1) at both ends of the range."""
+    return ((bits.astype(np.uint32) >> 9).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 8388608.0)
+
+
+def gumbel_from_bits(bits: np.ndarray) -> np.ndarray:
+    u = uniform_from_bits(bits)
+    return -np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+
+
 def gumbel_noise(key0: int, key1: int, position: int, vocab: int) -> torch.Tensor:
     """The Gumbel noise the sampling kernel adds to entry v: counter (v // 4, position, 0, 0), lane v % 4."""
     groups = (vocab + 3) // 4
@@ -54,8 +64,7 @@ def gumbel_noise(key0: int, key1: int, position: int, vocab: int) -> torch.Tenso
     z = np.zeros(groups, dtype=np.uint64)
     outs = philox4x32_10(g, z + np.uint64(position & 0xFFFFFFFF), z, z, key0 & 0xFFFFFFFF, key1 & 0xFFFFFFFF)
     bits = np.stack(outs, axis=1).reshape(-1)[:vocab].astype(np.uint32)
-    u = ((bits >> 8).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 16777216.0)
-    return torch.from_numpy(-np.log(-np.log(u, dtype=np.float32), dtype=np.float32))
+    return torch.from_numpy(gumbel_from_bits(bits))
 
 
 class EmulatedKernels:

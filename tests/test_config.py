@@ -46,6 +46,7 @@ def test_round_trip_through_a_folder(tmp_path):
     ({"n_layer": 0}, "positive integer"),
     ({"layer_norm_epsilon": 0.0}, "layer_norm_epsilon"),
     ({"n_inner": -4}, "n_inner"),
+    ({"scale_attn_weights": False}, "scale_attn_weights"),
 ])
 def test_bad_configs_are_refused(patch, match):
     with pytest.raises(ConfigError, match=match):

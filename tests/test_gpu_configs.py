@@ -41,6 +41,17 @@ def test_a_model_without_biases(dtype):
     check_all_cuttings("no biases", raw, 5, dtype, [70, 45, 100, 37])
 
 
+def test_a_head_size_of_40_runs_in_32_bit_and_is_refused_in_bfloat16():
+    """n_embd=320 with 8 heads: head size 40, a multiple of 8 and not of 16. The 32-bit path takes it (the cache keeps keys
+    in chunks of 8 head dimensions); bfloat16 needs steps of 16 and says so."""
+    raw = dict(TINY_A, n_embd=320, n_head=8, n_inner=None, n_positions=140)
+    check_all_cuttings("head size 40", raw, 6, "float32", [70, 45, 100, 37])
+    d = write_model(raw, 6, torch.bfloat16)
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "bfloat16", "--out",
+                        tempfile.mkdtemp(prefix="lev_trace_"), "--max-tokens", "64"], input="", capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "head_dim=40 must be a multiple of 16" in p.stderr
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_reference_s_schedules_through_trace_run(dtype):
     """The step schedules of the reference's paged-attention tests (tests/inference/test_paged_attention.py:293-442):

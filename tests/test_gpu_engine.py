@@ -768,6 +768,74 @@ def test_decode_steps_replayed_from_a_hip_graph_equal_eager_steps(dtype, monkeyp
     assert all(r.cache.groups[0].pool.n_free < 40 for r, _ in runners)
 
 
+def test_more_step_shapes_than_graphs_are_kept(monkeypatch):
+    """At most ``MAX_GRAPHS`` shapes are remembered; one more and every recorded graph is dropped (its shape is recorded
+    again when it comes twice more). With room for 3 and a block-table width that changes every 16 tokens, 110 decode
+    steps of two requests cross the limit several times and still equal the same steps run eagerly, bit for bit."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import load_model, make_cache
+    import levanter_amd.engine.step as step_mod
+
+    monkeypatch.setattr(step_mod, "GRAPH_BLOCK_BUCKET", 1)
+    monkeypatch.setattr(step_mod, "MAX_GRAPHS", 3)
+    d = write_model(TINY_A, 0, torch.bfloat16)
+    env = _env("bfloat16")
+    _, model = load_model(d, env)
+    cfg = InferenceEngineConfig(max_pages=24, max_seqs=4, page_size=16, max_pages_per_seq=8, compute_dtype="bfloat16")
+    runners = []
+    for graphs in (True, False):
+        cache = make_cache(model, cfg)
+        runners.append((ModelRunner(model, cache, env, use_graphs=graphs), cache))
+    g = torch.Generator().manual_seed(2)
+    toks = {k: torch.randint(0, 512, (128,), generator=g).tolist() for k in "ab"}
+    handles = [{k: c.open(k) for k in "ab"} for _, c in runners]
+    for (r, _), h in zip(runners, handles):
+        r.step([StepEntry(h["a"], toks["a"][:9], []), StepEntry(h["b"], toks["b"][:2], [])])
+    most, dropped, recorded_before = 0, 0, 0
+    for i in range(110):
+        outs = []
+        for (r, _), h in zip(runners, handles):
+            outs.append(r.step([StepEntry(h[k], [toks[k][h[k].length]], [0]) for k in "ab"]).cpu())
+        torch.testing.assert_close(outs[0], outs[1], rtol=0, atol=0, msg=lambda m: f"decode step {i}: {m}")
+        graphs = runners[0][0]._graphs
+        recorded = sum(1 for v in graphs.values() if v != "seen")
+        dropped += recorded < recorded_before
+        recorded_before = recorded
+        most = max(most, len(graphs))
+    assert dropped >= 1 and most <= 4, (dropped, most)
+
+
+def test_cache_sized_from_the_free_memory_of_the_device():
+    """``max_pages="auto"`` with the real query: the pool takes what is free once the weights are there, less the reserve,
+    capped at ``max_seqs * max_pages_per_seq``; a generation runs in it."""
+    from levanter_amd.cache.sizing import GIB, group_page_bytes
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import InferenceEngine, Request
+
+    d = write_model(TINY_B, 1, torch.bfloat16)
+    free_before, total = torch.cuda.mem_get_info(torch.device(DEV))
+    # a reserve that leaves about 1 GiB: far fewer pages than the cap, so the free memory is what decides
+    reserve = max(0.0, free_before / GIB - 1.0)
+    cfg = InferenceEngineConfig(max_pages="auto", cache_memory_reserve_gib=reserve, max_seqs=4096, max_pages_per_seq=256,
+                                page_size=16, compute_dtype="bfloat16")
+    engine = InferenceEngine.from_pretrained(d, cfg)
+    (group,) = engine.cache.groups
+    page_bytes = group_page_bytes(group.requirement, len(group.units), 16, 2)
+    n = group.pool.n_pages
+    assert 256 <= n < 4096 * 256
+    assert n * page_bytes <= free_before - reserve * GIB
+    assert n * page_bytes >= 0.5 * GIB, "about 1 GiB was on offer"
+    assert group.k_pages.shape[1] == n and group.k_pages.is_cuda
+    assert group.k_pages.numel() * 2 * 2 == n * page_bytes  # keys and values, two bytes an element
+    res = engine.generate([Request(prompt_tokens=[1, 2, 3, 4, 5], request_id=0, max_new_tokens=6)])
+    assert len(res.tokens[0]) == 6
+    # and with a reserve larger than the device there is nothing to promise
+    with pytest.raises(MemoryError, match="auto"):
+        InferenceEngine.from_pretrained(d, InferenceEngineConfig(max_pages="auto", cache_memory_reserve_gib=total / GIB + 1,
+                                                                  compute_dtype="bfloat16"))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graphed_decode_batches_are_filled_up_with_ghost_tokens(dtype):
     """Requests end one by one: 7, 6 and 5 live requests all run the graph of 8 rows, the missing ones being ghost

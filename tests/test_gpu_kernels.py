@@ -275,13 +275,13 @@ def test_row_counts_of_one_bucket_share_the_kernel_that_timing_chose(K, monkeypa
         assert float((h.double() - want).abs().max() / want.abs().max()) < 2e-2, M
 
 
-@pytest.mark.parametrize("M,K_,N,rows", [(64, 4096, 4096, None), (100, 16384, 4096, [99, 3, 3, 50]), (33, 8192, 1608, None),
+@pytest.mark.parametrize("M,K_,N,rows", [(64, 4096, 4096, None), (100, 16384, 4096, [99] + [3] * 40 + [50, 3]), (33, 8192, 1608, None),
                                          (300, 6400, 1600, [299, 0]), (64, 4096, 4104, None), (40, 8192, 8200, None),
                                          (16, 24576, 6144, [15, 0, 7]), (8, 24576, 6144, None)])
 def test_a_product_that_leaves_its_ranges_to_the_norm(K, M, K_, N, rows):
     """Where the product into the residual stream splits its sum over K into ranges, it may stop after writing them; the
-    norm that follows adds them to its rows, stores the rows back and normalises them in one kernel. The residual and
-    is bit for bit that of the finished product, the normed rows are those of the plain norm (up to the order in which the
+    norm that follows adds them to its rows, stores the rows back (unless it was given a selection of rows) and normalises
+    them in one kernel. The residual is bit for bit that of the finished product, the normed rows are those of the plain norm (up to the order in which the
     statistics are summed), for all rows and for a selection, also at a width where the norm falls back to finishing the product first (more than 8,192 columns)."""
     a = _rand(M, K_, dtype=torch.bfloat16, seed=M).to(DEV)
     w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=N).to(DEV)
@@ -305,10 +305,16 @@ def test_a_product_that_leaves_its_ranges_to_the_norm(K, M, K_, N, rows):
     # the fused kernel sums the row's statistics over 1,024 threads, the plain one over 256: one bfloat16 step at most
     assert float((h.float() - h_ref.float()).abs().max()) <= 2.0 ** -7 * float(h_ref.float().abs().max())
     assert float((h != h_ref).float().mean()) < 1e-3
-    touched = slice(None) if rows is None or N > 8192 else torch.tensor(sorted(set(rows)), device=DEV)
-    assert torch.equal(x[touched], x_ref[touched])
-    want = x0.double() + a.double() @ w.double().t() + bias.double()
-    assert float((x[touched].double() - want[touched]).abs().max() / want.abs().max()) < 2e-3
+    if rows is None or N > 8192:  # all rows (or no fused kernel at this width): the residual stream is finished
+        assert torch.equal(x, x_ref)
+        want = x0.double() + a.double() @ w.double().t() + bias.double()
+        assert float((x.double() - want).abs().max() / want.abs().max()) < 2e-3
+    else:  # a selection: nothing is stored back, so a row that is named twice is read as it was by both of its workgroups
+        assert torch.equal(x, x0)
+        for i, r in enumerate(rows):
+            for j in range(i + 1, len(rows)):
+                if rows[j] == r:
+                    assert torch.equal(h[i], h[j])
     # finishing it by itself gives the same residual
     x2 = x0.clone()
     K.finish(K.linear(a, w, bias, x2, residual=x2, may_leave_pending=True))
@@ -640,6 +646,24 @@ def test_sample_ties_and_frequencies(K):
     # the noise is the documented function of (key, position, entry)
     noise = gumbel_noise(3, 12345, 0, 5)
     assert int(toks[3]) == int(torch.argmax(base / t + noise))
+
+
+def test_sample_where_the_random_bits_are_all_ones(K):
+    """Key (1, 5), position 522: entry 21194 of a 50,257-entry vocabulary draws the largest value the generator has. Its
+    noise is the largest possible, about 16.6, and finite: an entry 30 above the rest still wins, and among equal logits
+    that entry wins, as the plain statement of the noise says."""
+    V = 50257
+    keys = torch.tensor([[1, 5], [1, 5]], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([522, 522], dtype=torch.int32, device=DEV)
+    logits = torch.zeros(2, V)
+    logits[0, 7] = 30.0
+    toks = torch.empty(2, dtype=torch.int32, device=DEV)
+    lps = torch.empty(2, device=DEV)
+    K.sample(logits.to(DEV), torch.ones(2, device=DEV), keys, pos, toks, lps)
+    assert toks.cpu().tolist() == [7, 21194]
+    assert bool(torch.isfinite(lps).all())
+    noise = gumbel_noise(1, 5, 522, V)
+    assert int(torch.argmax(noise)) == 21194 and bool(torch.isfinite(noise).all())
 
 
 @pytest.mark.parametrize("H,KVH,HD,PS,kv_lens,window", [

@@ -325,3 +325,16 @@ def test_warm_up_meets_the_row_counts_of_serving():
     shapes = {(len(b), sum(b)) for b in model.batches}
     assert {(1, 32), (1, 256), (64, 64), (32, 32), (2, 257)} <= shapes, sorted(shapes)
     assert engine.scheduler.idle and all_released(engine)
+
+
+def test_warm_up_fills_a_step_s_budget_with_several_prompts_when_one_request_cannot_hold_it():
+    """``max_prefill_size`` is a step's budget, ``page_size * max_pages_per_seq`` a request's limit: where the budget is
+    larger (the 20B workload: 2,048 prompt tokens a step, requests of 1,552), serving runs steps of several prompts, and
+    the ladder has to reach their row counts."""
+    engine, model = make_engine(max_pages=256, max_seqs=8, max_pages_per_seq=4, max_prefill_size=150, max_seqs_in_prefill=4)
+    engine.warm_up()
+    sums = {sum(b) for b in model.batches}
+    assert 150 in sums and 63 in sums, sorted(sums)
+    assert any(sum(b) == 150 and b == [63, 63, 24] for b in model.batches)
+    assert any(len(b) > 3 and sum(b) > 150 for b in model.batches), "a whole budget beside decoding requests"
+    assert engine.scheduler.idle and all_released(engine)
