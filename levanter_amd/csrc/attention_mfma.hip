@@ -75,10 +75,40 @@ __device__ __forceinline__ float max_over_lane_groups(float v) {
 // scale_log2 = scale * log2(e): scores, maxima and sums live in the base-2 domain, exp is the bare v_exp_f32.
 // q_pos: position of this lane's query row (or -1 for a padding row); key0: position of key 0 of the block.
 // need_mask (wave-uniform): false when every key of the block is visible to every row of the tile.
+// hook (wave-uniform, off by default): what a model may do to a score between the scaling and the mask
+// (src/levanter/layers/attention.py:361-367): add a term that depends on the head and on the distance between query and
+// key (bias_row: this lane's head's row of a float32 table [heads][bias_len], distances beyond it take its last entry),
+// then cap it softly, cap * tanh(score / cap). Both in natural units, before the change to base 2.
+struct ScoreHook {
+  float scale;           // the plain scale (scale_log2 / log2(e))
+  float softcap;         // 0: none
+  const float* bias_row; // null: none
+  int bias_len;
+};
+__device__ __forceinline__ float hooked_score(float raw, const ScoreHook& hk, int q_pos, int kp) {
+  float s = raw * hk.scale;
+  if (hk.bias_row) s += hk.bias_row[min(max(q_pos - kp, 0), hk.bias_len - 1)];
+  if (hk.softcap > 0.f) s = hk.softcap * tanhf(s / hk.softcap);
+  return s * 1.4426950408889634f;
+}
 __device__ __forceinline__ void softmax_block(f32x4 st[2][2], float scale_log2, int q_pos, int lo, int key0, int g,
-                                              bool need_mask, float& m, float& l, f32x4* o, u32x4 pf[2]) {
+                                              bool need_mask, float& m, float& l, f32x4* o, u32x4 pf[2], bool hook = false,
+                                              const ScoreHook* hk = nullptr) {
   float mx = -INFINITY;
-  if (need_mask) {
+  if (hook) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kp = key0 + 32 * u + 8 * g + 4 * h + r;
+          const bool ok = kp <= q_pos && kp >= lo;
+          const float s = ok ? hooked_score(st[u][h][r], *hk, q_pos, kp) : -INFINITY;
+          st[u][h][r] = s;
+          mx = fmaxf(mx, s);
+        }
+  } else if (need_mask) {
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -199,11 +229,14 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
                                              const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                                              const int* __restrict__ positions, const int* __restrict__ token_seq,
                                              const int* __restrict__ block_tables, int bt_stride, int t0, int rows, int h,
-                                             int H, int KVH, int ps_shift, float scale, int window, KsPtr Ks, VsPtr Vs) {
+                                             int H, int KVH, int ps_shift, float scale, int window, float softcap,
+                                             const float* __restrict__ score_bias, int bias_len, KsPtr Ks, VsPtr Vs) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int fr = lane & 15, g = lane >> 4;
   const int kvh = h / (H / KVH);
   const float scale_log2 = scale * 1.4426950408889634f;
+  const bool hook = softcap > 0.f || score_bias != nullptr;
+  const ScoreHook hk = {scale, softcap, score_bias ? score_bias + (size_t)h * bias_len : nullptr, bias_len};
   const int pos0 = positions[t0];
   const int* bt = block_tables + (size_t)token_seq[t0] * bt_stride;
   const int wave_row0 = wave * PF_QT * 16;
@@ -380,7 +413,7 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
     // and an order of issue given to the compiler. Left alone it emits each part by itself, every product behind a wait
     // for its own LDS read.
     const int p_first = pos0 + wave_row0, p_last = p_first + (PF_QT - 1) * 16 + 15;
-    if (n_qt == PF_QT && key0 + 63 <= p_first && (window <= 0 || p_last - window + 1 <= key0) && key0 + 127 <= hi) {
+    if (!hook && n_qt == PF_QT && key0 + 63 <= p_first && (window <= 0 || p_last - window + 1 <= key0) && key0 + 127 <= hi) {
       bool all[PF_QT];
       float m_cand[PF_QT];
       bool raise = false;
@@ -446,7 +479,7 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
         if (live[qt]) {
           const int p0 = pos0 + wave_row0 + qt * 16;  // first row of the tile: does it see the whole block, and the last row too
           const bool need_mask = !(key0 + 63 <= p0 && (window <= 0 || p0 + 15 - window + 1 <= key0));
-          softmax_block(st[qt], scale_log2, q_pos[qt], lo[qt], key0, g, need_mask, m[qt], l[qt], o[qt], pf[qt]);
+          softmax_block(st[qt], scale_log2, q_pos[qt], lo[qt], key0, g, need_mask, m[qt], l[qt], o[qt], pf[qt], hook, &hk);
         }
     }
     stage_k(cur);              // K(kb + 2) over K(kb), which the iteration before read
@@ -495,7 +528,8 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
                           const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                           const int* __restrict__ positions, const int* __restrict__ token_seq,
                           const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int n_tiles, int pair,
-                          int H, int KVH, int ps_shift, float scale, int window) {
+                          int H, int KVH, int ps_shift, float scale, int window, float softcap,
+                          const float* __restrict__ score_bias, int bias_len) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][4][NCHUNK][16][8];  // [buffer][score tile 2u+h][chunk][row][8]
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][VS_STRIDE];
   // Workgroups go to the 8 XCDs in turn, each with an L2 of its own. A kv head's keys and values are read by every tile
@@ -514,10 +548,10 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
   }
   const int first = x, second = n_tiles - 1 - x;
   prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * first],
-               tiles[2 * first + 1], h, H, KVH, ps_shift, scale, window, Ks, Vs);
+               tiles[2 * first + 1], h, H, KVH, ps_shift, scale, window, softcap, score_bias, bias_len, Ks, Vs);
   if (pair && second > first)
     prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * second],
-                 tiles[2 * second + 1], h, H, KVH, ps_shift, scale, window, Ks, Vs);
+                 tiles[2 * second + 1], h, H, KVH, ps_shift, scale, window, softcap, score_bias, bias_len, Ks, Vs);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -541,7 +575,8 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
                          const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
                          const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
                          float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
-                         int H, int KVH, int ps_shift, int splits, float scale, int window, int wg_merge) {
+                         int H, int KVH, int ps_shift, int splits, float scale, int window, int wg_merge, float softcap,
+                         const float* __restrict__ score_bias, int bias_len) {
   const int PS = 1 << ps_shift, ps_mask = PS - 1;
   const float scale_log2 = scale * 1.4426950408889634f;
   const int lane = threadIdx.x & 63;
@@ -557,6 +592,8 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   const int kb_begin = kb_first + z * per, kb_end = min(kb_last + 1, kb_begin + per);
   const int head = kvh * G + fr;  // this lane's query head (column of Q^T)
   const int q_pos = fr < G ? pos : -1;
+  const bool hook = softcap > 0.f || score_bias != nullptr;
+  const ScoreHook hk = {scale, softcap, score_bias ? score_bias + (size_t)min(head, H - 1) * bias_len : nullptr, bias_len};
   const size_t head_elems = (size_t)HD << ps_shift;
   const bool fused = k_new != nullptr;
   // The new key and value are copied to their page by one wave of the (token, kv head): the last one if it has no keys
@@ -696,7 +733,7 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
         st[u][hh] = acc;
       }
     u32x4 pf[2];
-    softmax_block(st, scale_log2, q_pos, lo, key0, g, key0 + 63 > pos || key0 < lo, m, l, o, pf);
+    softmax_block(st, scale_log2, q_pos, lo, key0, g, key0 + 63 > pos || key0 < lo, m, l, o, pf, hook, &hk);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -799,7 +836,8 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
                                                const int* block_tables, int bt_stride, const int* prefill_tiles,
                                                int n_prefill_tiles, const int* decode_tokens, int n_decode, const void* k_new,
                                                const void* v_new, long kv_stride, const int* dest, void* workspace, int H,
-                                               int KVH, int PS, int splits, float scale, int window, hipStream_t stream) {
+                                               int KVH, int PS, int splits, float scale, int window, float softcap,
+                                               const float* score_bias, int bias_len, hipStream_t stream) {
   int ps_shift = 0;
   while ((1 << ps_shift) < PS) ++ps_shift;
   if ((1 << ps_shift) != PS) return lev_fail("attention (matrix cores): page_size=%d must be a power of two", PS);
@@ -810,7 +848,7 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     LEV_NAME(attn_prefill_hd)<<<grid, PF_THREADS, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
                                                         (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq,
                                                         block_tables, bt_stride, prefill_tiles, n_prefill_tiles, pair, H,
-                                                        KVH, ps_shift, scale, window);
+                                                        KVH, ps_shift, scale, window, softcap, score_bias, bias_len);
     if (int rc = lev_check_launch("attention prefill")) return rc;
   }
   if (n_decode > 0) {
@@ -826,7 +864,7 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
     LEV_NAME(attn_decode_hd)<<<grid, wg_merge ? 64 * splits : 64, wg_merge ? merge_bytes : 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, positions, token_seq, block_tables,
         bt_stride, decode_tokens, (const bf16_t*)k_new, (const bf16_t*)v_new, kv_stride, dest, ws_m, ws_l, ws_o, H, KVH, ps_shift,
-        splits, scale, window, wg_merge);
+        splits, scale, window, wg_merge, softcap, score_bias, bias_len);
     if (int rc = lev_check_launch("attention decode")) return rc;
     if (splits > 1 && !wg_merge) {
       dim3 cgrid(n_decode, H);

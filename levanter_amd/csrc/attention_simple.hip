@@ -17,7 +17,8 @@ __global__ void __launch_bounds__(64)
 attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long o_stride,
                         const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ positions,
                         const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride, int H,
-                        int KVH, int HD, int PS, float scale, int window) {
+                        int KVH, int HD, int PS, float scale, int window, float softcap, const float* __restrict__ score_bias,
+                        int bias_len) {
   __shared__ float qs[AS_MAX_HD];
   __shared__ float ps[64];
   __shared__ int pg[64];
@@ -46,6 +47,10 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
       const T* kb = k_pages + ((size_t)page * KVH + kvh) * head_elems;
       float dot = 0.f;
       for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_float<T>(kb[((size_t)(d >> 3) * PS + off) * 8 + (d & 7)]), dot);
+      // between the scaling and the mask a model may add a term per (head, distance) and cap the score softly
+      // (src/levanter/layers/attention.py:361-367); both are off unless asked for
+      if (score_bias) dot += score_bias[(size_t)h * bias_len + min(pos - kp, bias_len - 1)];
+      if (softcap > 0.f) dot = softcap * tanhf(dot / softcap);
       s = dot;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -85,23 +90,26 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 extern "C" int lev_attention_simple(const void* q, long q_stride, void* out, long o_stride, const void* k_pages,
                                     const void* v_pages, const int* positions, const int* token_seq, const int* block_tables,
                                     int bt_stride, int T, int H, int KVH, int HD, int PS, float scale, int window, int dtype,
-                                    hipStream_t stream) {
+                                    float softcap, const float* score_bias, int bias_len, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(HD > 0 && HD % 8 == 0 && HD <= AS_MAX_HD, "attention: head_dim=%d must be a multiple of 8 and at most %d", HD,
               AS_MAX_HD);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(H <= 65535, "attention: too many heads (%d)", H);
   LEV_REQUIRE(window >= 0, "attention: window=%d must not be negative", window);
+  LEV_REQUIRE(softcap >= 0.f && (!score_bias || bias_len >= 1), "attention: soft cap %g must not be negative and a bias table needs entries (%d)",
+              (double)softcap, bias_len);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "attention: unknown dtype %d", dtype);
   if (T == 0) return 0;
   dim3 grid(T, H);
   if (dtype == LEV_F32)
     attention_simple_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_stride, (float*)out, o_stride,
                                                            (const float*)k_pages, (const float*)v_pages, positions, token_seq,
-                                                           block_tables, bt_stride, H, KVH, HD, PS, scale, window);
+                                                           block_tables, bt_stride, H, KVH, HD, PS, scale, window, softcap, score_bias, bias_len);
   else
     attention_simple_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, o_stride,
                                                             (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions,
-                                                            token_seq, block_tables, bt_stride, H, KVH, HD, PS, scale, window);
+                                                            token_seq, block_tables, bt_stride, H, KVH, HD, PS, scale, window, softcap, score_bias,
+                                                            bias_len);
   return lev_check_launch("attention_simple");
 }

@@ -13,6 +13,7 @@ unit only when it has no library or the sources changed; ``build`` builds every 
 """
 from __future__ import annotations
 
+import ctypes
 import hashlib
 import os
 import shutil
@@ -21,6 +22,7 @@ import sys
 import tempfile
 import time
 from concurrent.futures import ThreadPoolExecutor
+from dataclasses import dataclass, field
 from typing import Dict, Iterable, List, Optional, Tuple
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -29,25 +31,50 @@ ARCH = "gfx950"
 
 MFMA_ATTENTION_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
 
-# unit -> [(source, extra defines, object name)]
-UNITS: Dict[str, List[Tuple[str, List[str], str]]] = {
-    "core": [
-        ("errors.hip", [], "errors.o"),
-        ("elementwise.hip", [], "elementwise.o"),
-        ("gemm_simple.hip", [], "gemm_simple.o"),
-        ("attention_simple.hip", [], "attention_simple.o"),
-        ("attention_common.hip", [], "attention_common.o"),
-    ],
-    "gemm_mfma": [("gemm_mfma.hip", [], "gemm_mfma.o")],
-    "gemm_library": [("gemm_library.hip", [], "gemm_library.o")],
-}
-# libraries a unit is linked against
-UNIT_LINK_FLAGS: Dict[str, List[str]] = {"gemm_library": ["-lhipblaslt"]}
-for _hd in MFMA_ATTENTION_HEAD_DIMS:
-    UNITS[f"attn_hd{_hd}"] = [
-        ("attention_mfma.hip", [f"-DLEV_HD={_hd}"], f"attention_mfma_hd{_hd}.o"),
-        ("attention_dispatch.hip", [f"-DLEV_HD={_hd}"], f"attention_dispatch_hd{_hd}.o"),
-    ]
+
+@dataclass
+class KernelUnit:
+    """One shared library: its sources, how they are compiled and linked, and the ``extern "C"`` entry points it offers.
+
+    ``sources``: (file, extra defines, object name); a relative file lies in ``source_dir``. Sources may include the
+    headers of ``csrc/`` (``common.h``: the error functions, dtype tags, reductions) wherever they lie themselves.
+    ``signatures``: entry point -> ctypes argument types; the result is an int (0, or a negative code with a message in
+    ``lev_last_error()``) unless the name ends in ``_workspace`` (a byte count). ``HipKernels`` sets them when it
+    loads the library."""
+
+    name: str
+    sources: List[Tuple[str, List[str], str]]
+    source_dir: str = CSRC
+    link_flags: List[str] = field(default_factory=list)
+    signatures: Dict[str, list] = field(default_factory=dict)
+
+    def source_path(self, src: str) -> str:
+        return src if os.path.isabs(src) else os.path.join(self.source_dir, src)
+
+
+UNITS: Dict[str, KernelUnit] = {}
+
+
+def register_unit(name: str, sources, *, source_dir: str = CSRC, link_flags: Iterable[str] = (), signatures: Optional[Dict[str, list]] = None,
+                  replace: bool = False) -> KernelUnit:
+    """Make a kernel library known: ``ensure_built(name)`` compiles it when it is missing or stale and
+    ``HipKernels.call(name, entry, ...)`` loads it at its first use. A part that brings a kernel of its own registers a unit
+    for it from its own module (its ``.hip`` may lie anywhere); nothing in this package has to change.
+    ``sources``: file names, or (file, defines, object name) where one file is compiled several ways."""
+    if name in UNITS and not replace:
+        raise ValueError(f"kernel unit {name!r} is already registered")
+    items = []
+    for src in sources:
+        if isinstance(src, str):
+            src = (src, [], os.path.splitext(os.path.basename(src))[0] + ".o")
+        items.append((src[0], list(src[1]), src[2]))
+    unit = KernelUnit(name, items, source_dir, list(link_flags), dict(signatures or {}))
+    UNITS[name] = unit
+    return unit
+
+
+def unregister_unit(name: str) -> None:
+    UNITS.pop(name, None)
 
 
 def attention_unit(head_dim: int) -> str:
@@ -80,36 +107,39 @@ def find_hipcc() -> Optional[str]:
     return None
 
 
-def _with_includes(names: Iterable[str]) -> List[str]:
-    """The given sources and every file of ``csrc/`` that they include with ``#include "..."``, directly or not."""
-    seen, todo = set(), list(names)
+def _with_includes(unit: KernelUnit) -> List[str]:
+    """The unit's sources and every file that they include with ``#include "..."``, directly or not: looked up beside the
+    including file and in ``csrc/`` (the include path of every compilation)."""
+    seen, todo = set(), [unit.source_path(src) for src, _, _ in unit.sources]
     while todo:
-        name = todo.pop()
-        if name in seen:
+        path = todo.pop()
+        if path in seen:
             continue
-        seen.add(name)
-        with open(os.path.join(CSRC, name), encoding="utf-8") as f:
+        seen.add(path)
+        with open(path, encoding="utf-8") as f:
             for line in f:
                 line = line.strip()
                 if line.startswith("#include \""):
                     inc = line.split('"')[1]
-                    if os.path.isfile(os.path.join(CSRC, inc)):
-                        todo.append(inc)
+                    for base in (os.path.dirname(path), CSRC):
+                        if os.path.isfile(os.path.join(base, inc)):
+                            todo.append(os.path.join(base, inc))
+                            break
     return sorted(seen)
 
 
 def source_hash(unit: str = "core") -> str:
     """Hash of what a unit is built from: the flags, its own sources and defines, and the headers they include."""
+    u = UNITS[unit]
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    names = _with_includes(src for src, _, _ in UNITS[unit])
-    for name in names:
-        h.update(name.encode())
-        with open(os.path.join(CSRC, name), "rb") as f:
+    for path in _with_includes(u):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
             h.update(f.read())
-    for _, defines, obj in UNITS[unit]:
+    for _, defines, obj in u.sources:
         h.update((" ".join(defines) + obj).encode())
-    h.update(" ".join(UNIT_LINK_FLAGS.get(unit, [])).encode())
+    h.update(" ".join(u.link_flags).encode())
     return h.hexdigest()[:16]
 
 
@@ -165,7 +195,7 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
         return paths
     obj_dir = os.path.join(library_dir(), "_build")
     os.makedirs(obj_dir, exist_ok=True)
-    items = [item for u in todo for item in UNITS[u]]
+    items = [(UNITS[u], item) for u in todo for item in UNITS[u].sources]
     jobs = jobs or min(8, os.cpu_count() or 1, len(items))
     env = dict(os.environ)
     home = env.get("HOME", "")
@@ -174,10 +204,10 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
     t0 = time.time()
     _log(f"compiling {len(items)} HIP objects ({', '.join(todo)}) for {ARCH} with {jobs} jobs ...")
 
-    def compile_one(item) -> None:
-        src, defines, obj_name = item
-        obj = os.path.join(obj_dir, obj_name)
-        cmd = [hipcc, *HIPCC_FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
+    def compile_one(unit_item) -> None:
+        unit, (src, defines, obj_name) = unit_item
+        obj = os.path.join(obj_dir, _object_name(unit, obj_name))
+        cmd = [hipcc, *HIPCC_FLAGS, f"-I{CSRC}", *defines, "-c", unit.source_path(src), "-o", obj]
         t = time.time()
         r = subprocess.run(cmd, capture_output=True, text=True, env=env)
         if r.returncode != 0:
@@ -188,9 +218,9 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
         list(pool.map(compile_one, items))
     for u in todo:
         lib = paths[u]
-        objs = [os.path.join(obj_dir, obj_name) for _, _, obj_name in UNITS[u]]
+        objs = [os.path.join(obj_dir, _object_name(UNITS[u], obj_name)) for _, _, obj_name in UNITS[u].sources]
         tmp = lib + f".tmp{os.getpid()}"
-        r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs, *UNIT_LINK_FLAGS.get(u, [])],
+        r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs, *UNITS[u].link_flags],
                            capture_output=True, text=True, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed to link {lib_name(u)}:\n{_filter(r.stderr)}")
@@ -199,6 +229,11 @@ def build(force: bool = True, jobs: Optional[int] = None, units: Optional[Iterab
             f.write(source_hash(u))
     _log(f"built {', '.join(lib_name(u) for u in todo)} in {library_dir()} in {time.time() - t0:.0f}s")
     return paths
+
+
+def _object_name(unit: KernelUnit, obj_name: str) -> str:
+    """Objects of units outside ``csrc/`` carry the unit's name: two units may both have a ``kernel.o``."""
+    return obj_name if unit.source_dir == CSRC else f"{unit.name}__{obj_name}"
 
 
 def _filter(stderr: str) -> str:
@@ -214,3 +249,36 @@ def ensure_built(unit: str = "core") -> str:
         _log(f"warning: {lib} is older than its sources and hipcc is not there to rebuild it")
         return lib
     return build(force=True, units=[unit])[unit]
+
+
+# ---- the units of this package --------------------------------------------------------------------------------
+_P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+
+register_unit("core", ["errors.hip", "elementwise.hip", "gemm_simple.hip", "attention_simple.hip", "attention_common.hip"], signatures={
+    "lev_embed": [_P] * 5 + [_I, _I, _I, _P],
+    "lev_norm": [_P] * 5 + [_I, _I, _F, _I, _I, _P],
+    "lev_norm_pending": [_P, _P, _I] + [_P] * 5 + [_I, _I, _I, _F, _I, _I, _P],
+    "lev_kv_write": [_P, _P, _L, _L, _P, _P, _P] + [_I] * 5 + [_P],
+    "lev_sample": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "lev_sample_workspace": [_I],
+    "lev_feed_tokens": [_P, _P, _P, _I, _P],
+    "lev_linear_simple": [_P, _L, _P, _P, _P, _L, _P, _L] + [_I] * 6 + [_P],
+    "lev_attention_simple": [_P, _L, _P, _L, _P, _P, _P, _P, _P] + [_I] * 6 + [_F, _I, _I, _F, _P, _I, _P],
+    "lev_attention_mfma_workspace": [_I] * 5,
+})
+register_unit("gemm_mfma", ["gemm_mfma.hip"], signatures={
+    "lev_linear_mfma": [_P, _L, _P, _P, _P, _L, _P, _L, _P] + [_I] * 6 + [_P],
+    "lev_linear_mfma_workspace": [_I, _I, _I],
+    "lev_linear_mfma_ranges": [_I, _I, _I],
+    "lev_linear_mfma_finish": [_P, _P, _P, _L, _P, _L] + [_I] * 5 + [_P],
+})
+# the vendor library's GEMM (hipBLASLt) behind the same interface
+register_unit("gemm_library", ["gemm_library.hip"], link_flags=["-lhipblaslt"], signatures={
+    "lev_linear_library": [_P, _L, _P, _P, _P, _L, _P, _L, _P, _L] + [_I] * 5 + [_P],
+    "lev_linear_library_workspace": [],
+})
+for _hd in MFMA_ATTENTION_HEAD_DIMS:
+    register_unit(attention_unit(_hd), [("attention_mfma.hip", [f"-DLEV_HD={_hd}"], f"attention_mfma_hd{_hd}.o"),
+                                        ("attention_dispatch.hip", [f"-DLEV_HD={_hd}"], f"attention_dispatch_hd{_hd}.o")], signatures={
+        "lev_attention_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _L, _P, _P] + [_I] * 5 + [_F, _I, _F, _P, _I, _P],
+    })

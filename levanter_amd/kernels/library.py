@@ -89,19 +89,7 @@ class HipKernels:
         L = self.lib
         L.lev_last_error.restype = ctypes.c_char_p
         L.lev_abi_version.restype = c_int
-        self._set_signatures(L, {
-            "lev_embed": [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p],
-            "lev_norm": [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_int, c_void_p],
-            "lev_norm_pending": [c_void_p, c_void_p, c_int] + [c_void_p] * 5 + [c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
-            "lev_kv_write": [c_void_p, c_void_p, c_long, c_long, c_void_p, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p],
-            "lev_sample": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-            "lev_sample_workspace": [c_int],
-            "lev_feed_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_void_p],
-            "lev_linear_simple": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 6 + [c_void_p],
-            "lev_attention_simple": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
-            + [c_int] * 6 + [c_float, c_int, c_int, c_void_p],
-            "lev_attention_mfma_workspace": [c_int] * 5,
-        })
+        self._set_signatures(L, _build.UNITS["core"].signatures)
         self.use_mfma = os.environ.get("LEVANTER_AMD_NO_MFMA", "0") != "1"
         # the vendor library's GEMM for prompt-sized row counts (see use_library); "0" keeps every product on our kernels
         self.gemm_library = os.environ.get("LEVANTER_AMD_GEMM_LIBRARY", "1") != "0"
@@ -127,36 +115,37 @@ class HipKernels:
             fn.restype = c_long if name.endswith("_workspace") else c_int
 
     def _unit(self, unit: str):
-        """The library of a unit other than ``core``, built and loaded at its first use."""
+        """The library of a registered unit other than ``core``, built and loaded at its first use."""
         lib = self._units.get(unit)
         if lib is None:
+            if unit not in _build.UNITS:
+                raise KernelError(f"unknown kernel unit {unit!r}; registered: {', '.join(_build.UNITS)}")
             path = _build.ensure_built(unit)
             try:
                 lib = ctypes.CDLL(path)
             except OSError as e:
                 raise KernelError(f"the HIP library {path} cannot be loaded: {e}") from None
-            if unit == "gemm_library":
-                self._set_signatures(lib, {
-                    "lev_linear_library": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long]
-                    + [c_int] * 5 + [c_void_p],
-                    "lev_linear_library_workspace": [],
-                })
-            elif unit == "gemm_mfma":
-                self._set_signatures(lib, {
-                    "lev_linear_mfma": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p]
-                    + [c_int] * 6 + [c_void_p],
-                    "lev_linear_mfma_workspace": [c_int, c_int, c_int],
-                    "lev_linear_mfma_ranges": [c_int, c_int, c_int],
-                    "lev_linear_mfma_finish": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long] + [c_int] * 5 + [c_void_p],
-                })
-            else:
-                self._set_signatures(lib, {
-                    "lev_attention_mfma": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                           c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p]
-                    + [c_int] * 5 + [c_float, c_int, c_void_p],
-                })
+            self._set_signatures(lib, _build.UNITS[unit].signatures)
             self._units[unit] = lib
         return lib
+
+    def call(self, unit: str, entry: str, *args) -> None:
+        """Call an ``extern "C"`` entry point of a registered unit (``kernels.build.register_unit``): the way a part reaches
+        a kernel of its own. Arguments as the unit's signature says (``tensor_ptr(t)`` for a tensor's address,
+        ``stream()`` for the current HIP stream); the entry point returns 0, or a negative code with its message in
+        ``lev_last_error()`` (``LEV_REQUIRE`` of ``common.h``), which is raised as a ``KernelError``."""
+        lib = self.lib if unit == "core" else (self._units.get(unit) or self._unit(unit))
+        try:
+            fn = getattr(lib, entry)
+        except AttributeError:
+            raise KernelError(f"kernel unit {unit!r} has no entry point {entry!r}") from None
+        self._check(fn(*args))
+
+    tensor_ptr = staticmethod(lambda t: None if t is None else t.data_ptr())
+
+    def stream(self):
+        """The HIP stream that launches go to now (the current one, or the one held for a forward pass)."""
+        return self._s()
 
     def hold_stream(self) -> None:
         """Look the current stream up once and use it for every launch until ``release_stream``: a model's forward pass
@@ -366,9 +355,13 @@ class HipKernels:
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,
                         page_size: int, scale: float, window: Optional[int], block_tables, k_new=None, v_new=None,
-                        dest=None) -> bool:
+                        dest=None, softcap: Optional[float] = None, score_bias=None) -> bool:
         """Causal attention of the step's query tokens over the pages. ``meta`` is the step's
         ``AttentionMeta`` (positions, token_seq and the work lists), block_tables int32 [S, B].
+
+        ``score_bias`` (float32 ``[n_heads, L]``): entry ``[h, min(d, L - 1)]`` is added to the scaled score of head ``h``
+        for a key ``d`` positions behind its query; ``softcap``: scores become ``softcap * tanh(score / softcap)`` (after
+        the bias, before the mask). Both off by default.
 
         ``k_new``/``v_new``/``dest``: the step's new keys and values, not yet written. Returns True if this
         call has written them to their pages (a step of single tokens on the matrix-core path does it inside
@@ -404,6 +397,13 @@ class HipKernels:
                                       _ptr(meta.token_seq), _ptr(meta.prefill_tiles), _ptr(meta.decode_tokens), block_tables)
         mfma, splits, _ws, ws_ptr, lib, bt_ptr, bt_width, pos_ptr, seq_ptr, tiles_ptr, decode_ptr, _bt = plan
         w = int(window) if window else 0
+        cap = float(softcap) if softcap else 0.0
+        bias_len = 0
+        if score_bias is not None:
+            if not (score_bias.is_cuda and score_bias.dtype == torch.float32 and score_bias.dim() == 2 and score_bias.shape[0] == n_heads
+                    and score_bias.is_contiguous() and score_bias.shape[1] >= 1):
+                raise KernelError("attention: the score bias must be a contiguous float32 table [heads, distances] on the GPU")
+            bias_len = score_bias.shape[1]
         qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
         kvs = 0
         if k_new is not None:
@@ -421,11 +421,11 @@ class HipKernels:
                 _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, tiles_ptr,
                 meta.n_prefill_tiles, decode_ptr, meta.n_decode, _ptr(k_new), _ptr(v_new), kvs,
                 _ptr(dest) if k_new is not None else None, ws_ptr, n_heads, n_kv_heads, head_dim, page_size,
-                splits, float(scale), w, self._s()))
+                splits, float(scale), w, cap, _ptr(score_bias), bias_len, self._s()))
             return k_new is not None
         self._check(self.lib.lev_attention_simple(
             _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, T, n_heads, n_kv_heads,
-            head_dim, page_size, float(scale), w, _DT[dt], self._s()))
+            head_dim, page_size, float(scale), w, _DT[dt], cap, _ptr(score_bias), bias_len, self._s()))
         return False
 
     @staticmethod

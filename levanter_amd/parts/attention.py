@@ -35,6 +35,13 @@ class CausalSelfAttention(Mixer):
         self.head_dim = int(p["head_dim"])
         self.scale = float(p["scale"])
         self.window = p.get("window")
+        # what a model may do to a score between the scaling and the mask (src/levanter/layers/attention.py:361-367): a
+        # soft cap, and a term per head and distance from a float32 table [heads, distances] (the parameter ``score_bias``)
+        self.softcap = p.get("softcap")
+        bias = tensors.get("score_bias")
+        self.score_bias = None if bias is None else bias.to(env.device, torch.float32).contiguous()
+        if self.score_bias is not None and (self.score_bias.dim() != 2 or self.score_bias.shape[0] != self.n_heads):
+            raise ValueError(f"attention: the score bias must be [heads={self.n_heads}, distances], got {tuple(self.score_bias.shape)}")
         if self.n_heads % self.n_kv_heads != 0:
             raise ValueError(f"attention: {self.n_heads} heads are not a multiple of {self.n_kv_heads} key/value heads")
         # the cache keeps keys in chunks of 8 head dimensions; the matrix-core kernels need multiples of 16
@@ -68,6 +75,8 @@ class CausalSelfAttention(Mixer):
         a = ctx.empty(h.shape[0], self.q_cols)
         args = dict(n_heads=self.n_heads, n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, page_size=g.page_size,
                     scale=self.scale, window=self.window, block_tables=g.block_tables)
+        if self.softcap or self.score_bias is not None:
+            args.update(softcap=self.softcap, score_bias=self.score_bias)
         written = False
         if writes_cache:  # a step of single tokens writes the new keys and values inside the attention kernel
             written = ctx.kernels.paged_attention(q, a, unit.k_pages, unit.v_pages, ctx.attention, k_new=k, v_new=v,

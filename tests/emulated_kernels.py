@@ -136,7 +136,7 @@ class EmulatedKernels:
 
     # ---- attention
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads, n_kv_heads, head_dim, page_size, scale, window,
-                        block_tables, k_new=None, v_new=None, dest=None) -> bool:
+                        block_tables, k_new=None, v_new=None, dest=None, softcap=None, score_bias=None) -> bool:
         if k_new is not None:
             return False  # this stand-in never writes the cache inside attention: the caller calls kv_write
         T = q.shape[0]
@@ -150,6 +150,11 @@ class EmulatedKernels:
             ks = ks.float().repeat_interleave(g, 0)  # [H, n, hd]
             vs = vs.float().repeat_interleave(g, 0)
             s = torch.einsum("hd,hnd->hn", qt, ks)
+            if score_bias is not None:  # [heads, L]: entry min(distance, L - 1) of the head's row
+                dist = (pos - torch.arange(lo, pos + 1)).clamp(max=score_bias.shape[1] - 1)
+                s = s + score_bias.float().cpu()[:, dist]
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
             p = torch.softmax(s, -1)
             if q.dtype == torch.bfloat16:
                 p = p.to(torch.bfloat16).float()

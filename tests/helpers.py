@@ -78,3 +78,17 @@ def read_weights(model_dir: str, dtype=torch.float64) -> Dict[str, torch.Tensor]
     from safetensors.torch import load_file
 
     return {k: v.to(dtype) for k, v in load_file(os.path.join(model_dir, "model.safetensors")).items()}
+
+
+def toy_rotary_unit() -> str:
+    """The toy rotation's kernel (``toy_rotary.hip`` beside the tests) as a kernel unit of its own, registered with the
+    build from outside the package; returns the unit's name."""
+    import ctypes
+
+    from levanter_amd.kernels import build
+
+    if "toy_rotary" not in build.UNITS:
+        P_, I_, L_, F_ = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+        build.register_unit("toy_rotary", ["toy_rotary.hip"], source_dir=os.path.dirname(os.path.abspath(__file__)),
+                            signatures={"toy_rotate": [P_, L_, P_, I_, I_, I_, F_, I_, P_]})
+    return "toy_rotary"

@@ -10,7 +10,7 @@ import torch
 
 import plain_gpt2 as P
 from emulated_kernels import gumbel_noise
-from helpers import make_meta, read_weights, write_model
+from helpers import make_meta, read_weights, toy_rotary_unit, write_model
 from tiny_configs import TINY, TINY_A, TINY_B
 
 pytestmark = pytest.mark.gpu
@@ -883,12 +883,16 @@ def test_graphed_decode_batches_are_filled_up_with_ghost_tokens(dtype):
 
 
 def test_a_toy_rotary_position_encoding_registers_and_only_distances_count():
-    """Another position encoding, defined here: queries and keys are rotated by their absolute position before
-    the cache write (pairs (i, i + head_dim/2) of a head), the embedding adds no position. Compared with a plain
-    whole-sequence computation; and a shift of all positions changes nothing, because only distances count."""
+    """Another position encoding, defined here, with a kernel of its own: queries and keys are rotated by their absolute
+    position before the cache write (pairs (i, i + head_dim/2) of a head) by a HIP kernel that lies beside this test
+    (``toy_rotary.hip``), is registered as a kernel unit from here and is reached through ``kernels.call``; the embedding
+    adds no position. Compared with a plain whole-sequence computation; a shift of all positions changes nothing, because
+    only distances count; and the part is ``graph_safe``: the single-token steps are replayed from a HIP graph."""
+    from levanter_amd.kernels import KernelError
     from levanter_amd.parts import POSITION_ENCODINGS, PartSpec, PositionEncoding
 
     H, HD, BASE = 4, 16, 100.0
+    unit = toy_rotary_unit()
 
     def angles(pos):  # [T, HD/2]
         inv = BASE ** (-torch.arange(HD // 2, dtype=torch.float64) / (HD // 2))
@@ -902,18 +906,30 @@ def test_a_toy_rotary_position_encoding_registers_and_only_distances_count():
 
     @POSITION_ENCODINGS.register("toy_rotary")
     class ToyRotary(PositionEncoding):
-        graph_safe = True  # positions are read from device memory, shapes follow the step's sizes
+        graph_safe = True  # one kernel launch whose shape follows the step's sizes; positions are read from device memory
 
         def rotate(self, q, k, ctx):
-            pos = ctx.attention.positions.to(torch.float32)
-            inv = BASE ** (-torch.arange(HD // 2, dtype=torch.float32, device=q.device) / (HD // 2))
-            ang = pos[:, None] * inv[None, :]
-            c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
-            for t in (q, k):  # strided views into the fused projection's output: rotated in place, in 32-bit
-                v = t.view(t.shape[0], -1, HD) if t.is_contiguous() else t.unflatten(1, (-1, HD))
-                x1, x2 = v[..., : HD // 2].float().clone(), v[..., HD // 2:].float().clone()  # copies: float() of float32 is a view
-                v[..., : HD // 2] = (x1 * c - x2 * s_).to(t.dtype)
-                v[..., HD // 2:] = (x2 * c + x1 * s_).to(t.dtype)
+            kern = ctx.kernels
+            for t in (q, k):  # strided views into the fused projection's output: rotated in place
+                kern.call(unit, "toy_rotate", kern.tensor_ptr(t), t.stride(0), kern.tensor_ptr(ctx.attention.positions), t.shape[0],
+                          t.shape[1] // HD, HD, BASE, 0 if t.dtype == torch.float32 else 1, kern.stream())
+
+    # the kernel alone against the plain rotation, both dtypes, and its own error message through the package's channel
+    kern = _env("float32").kernels
+    pos = torch.tensor([0, 5, 130, 7], dtype=torch.int32, device=DEV)
+    for dt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        buf = torch.randn(4, 3 * H * HD, generator=torch.Generator().manual_seed(3)).to(dt).to(DEV)
+        view = buf[:, H * HD: 2 * H * HD]  # a strided view, as the keys are in the fused projection's output
+        want = plain_rotate(view.double().cpu().view(4, H, HD), pos.cpu()).view(4, -1)
+        kern.call(unit, "toy_rotate", kern.tensor_ptr(view), view.stride(0), kern.tensor_ptr(pos), 4, H, HD, BASE, 0 if dt == torch.float32 else 1,
+                  kern.stream())
+        torch.testing.assert_close(view.double().cpu(), want, rtol=tol, atol=tol)
+    with pytest.raises(KernelError, match="toy_rotate: bad sizes"):
+        kern.call(unit, "toy_rotate", kern.tensor_ptr(buf), buf.stride(0), kern.tensor_ptr(pos), 4, H, 15, BASE, 0, kern.stream())
+    with pytest.raises(KernelError, match="no entry point"):
+        kern.call(unit, "toy_rotate_backwards")
+    with pytest.raises(KernelError, match="unknown kernel unit"):
+        kern.call("no_such_unit", "f")
 
     try:
         d = write_model(TINY_A, 0, torch.float32)
@@ -945,8 +961,54 @@ def test_a_toy_rotary_position_encoding_registers_and_only_distances_count():
         for cuts in ([60], [23, 2, 30, 1, 1, 1, 1, 1]):
             got, _, _ = _run_cut(spec, t32, "float32", toks, cuts)
             torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=2e-5)
+        # replayed from a graph: the model says so, and the last single-token steps of the second cutting were replays
+        from levanter_amd.parts import DecoderLm
+
+        assert DecoderLm(spec, t32, _env("float32")).graph_safe
     finally:
         POSITION_ENCODINGS.unregister("toy_rotary")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_attention_description_with_a_soft_cap_and_a_score_bias(dtype):
+    """The attention part takes ``softcap`` and a ``score_bias`` tensor from its description (what
+    src/levanter/layers/attention.py:361-367 applies between scaling and mask) and hands them to the kernels: tiny A with
+    both in its second layer, whole and cut into portions and single tokens, against a plain whole-sequence computation."""
+    from levanter_amd.parts import TensorSpec
+
+    H, HD, CAP, L = 4, 16, 1.5, 12
+    d = write_model(TINY_A, 0, torch.float32 if dtype == "float32" else torch.bfloat16)
+    w = read_weights(d)
+    bias = -0.4 * torch.arange(L, dtype=torch.float64)[None, :] * torch.tensor([1.0, 0.5, 0.25, 2.0], dtype=torch.float64)[:, None]
+    tensors = {k: v.float() for k, v in w.items()}
+    tensors["h.1.attn.score_bias"] = bias.float()
+    spec = _toy_spec()
+    spec.layers[1].mixer.params["softcap"] = CAP
+    spec.layers[1].mixer.tensors["score_bias"] = TensorSpec("h.1.attn.score_bias", (H, L))
+    toks = torch.randint(0, 512, (50,), generator=torch.Generator().manual_seed(5)).tolist()
+    rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+    n = len(toks)
+    x = P.plain_embed(torch.tensor(toks), torch.arange(n), w["wte.weight"], w["wpe.weight"])
+    for i in range(2):
+        p = f"h.{i}."
+        hh = rounding(P.plain_layernorm(x, w[p + "ln_1.weight"], w[p + "ln_1.bias"], 1e-5))
+        q, k, v = P.plain_split_qkv(rounding(P.plain_linear(hh, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"])), H)
+        s = torch.einsum("htd,hsd->hts", q, k) / math.sqrt(HD)
+        if i == 1:
+            dist = (torch.arange(n)[:, None] - torch.arange(n)[None, :]).clamp(0, L - 1)
+            s = CAP * torch.tanh((s + bias[:, dist]) / CAP)
+        s = s.masked_fill(torch.arange(n)[None, :] > torch.arange(n)[:, None], float("-inf"))
+        o = rounding(torch.einsum("hts,hsd->htd", rounding(torch.softmax(s, -1)), v))
+        x = x + P.plain_linear(o.transpose(0, 1).reshape(n, -1), w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+        x = x + P.plain_mlp(rounding(P.plain_layernorm(x, w[p + "ln_2.weight"], w[p + "ln_2.bias"], 1e-5)), w, p, TINY_A, rounding)
+    want = rounding(P.plain_layernorm(x, w["ln_f.weight"], w["ln_f.bias"], 1e-5)) @ w["wte.weight"].T
+    plain_gpt2 = P.plain_logits(w, TINY_A, torch.tensor(toks))
+    assert float((want - plain_gpt2).abs().max()) > 0.05, "cap and bias must matter in this test"
+    run_tensors = tensors if dtype == "float32" else {k: (v if k.endswith("score_bias") else v.to(torch.bfloat16)) for k, v in tensors.items()}
+    tol = dict(rtol=1e-4, atol=2e-5) if dtype == "float32" else dict(rtol=2e-2, atol=8e-3)
+    for cuts in ([50], [20, 2, 19, 1, 1, 1, 1, 1, 1, 1, 1, 1]):
+        got, _, _ = _run_cut(spec, run_tensors, dtype, toks, cuts)
+        torch.testing.assert_close(got.double(), want, **tol)
 
 
 def test_a_toy_feed_forward_with_routing_registers_builds_and_steps():

@@ -503,6 +503,46 @@ def test_paged_attention(K, dtype, H, KVH, HD, PS, runs, window):
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KVH,HD,PS,runs,window", [
+    (4, 4, 64, 16, [(1, 300), (1, 17), (70, 150), (5, 5)], None),   # single tokens (split and merged), a later portion, a short prompt
+    (6, 2, 128, 16, [(130, 260), (1, 90)], 100),                    # query heads that share keys, a window
+    (3, 3, 48, 32, [(200, 200), (1, 1)], None),                     # most key blocks wholly before a tile's rows
+])
+@pytest.mark.parametrize("hook", ["softcap", "bias", "both"])
+def test_attention_scores_capped_softly_and_with_a_term_per_head_and_distance(K, dtype, H, KVH, HD, PS, runs, window, hook):
+    """Between the scaling and the mask a model may add a term that depends on head and distance and cap the scores
+    softly (src/levanter/layers/attention.py:361-367): both are arguments of the attention kernels, off by default. The
+    bias table is shorter than the longest distance (its last entry serves the rest) and steep enough, and the cap low
+    enough, that leaving either out, or applying them in the other order, changes the output by far more than the tolerance."""
+    kv_lens = [k for _, k in runs]
+    n_pages = sum((k + PS - 1) // PS for k in kv_lens) + 3
+    bt, kp, vp, kd, vd, ks, vs = _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed=9)
+    T = sum(q for q, _ in runs)
+    q = _rand(T, H * HD, dtype=dtype, seed=13, scale=3.0)
+    scale = 1 / math.sqrt(HD)
+    cap = 2.5 if hook in ("softcap", "both") else None
+    bias = None
+    if hook in ("bias", "both"):
+        slopes = torch.tensor([0.5 ** (h + 1) for h in range(H)])
+        bias = (-slopes[:, None] * torch.arange(40)[None, :].float() + 0.3 * _rand(H, 40, seed=4)).contiguous()
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=scale, window=window)
+    want = torch.empty(T, H * HD, dtype=dtype)
+    EMU.paged_attention(q, want, kp, vp, make_meta(runs, "cpu"), block_tables=bt, softcap=cap, score_bias=bias, **args)
+    plain = torch.empty(T, H * HD, dtype=dtype)
+    EMU.paged_attention(q, plain, kp, vp, make_meta(runs, "cpu"), block_tables=bt, **args)
+    assert float((want.float() - plain.float()).abs().max()) > 0.1, "the hook must matter in this test"
+    got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q.to(DEV), got, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), softcap=cap,
+                      score_bias=None if bias is None else bias.to(DEV), **args)
+    tol = dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    # and off again: the same launch without the arguments is the plain attention
+    got2 = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q.to(DEV), got2, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+    torch.testing.assert_close(got2.cpu().float(), plain.float(), **tol)
+
+
 def test_paged_attention_random_cases(K):
     """Forty random cases in bfloat16: head sizes 16 .. 128, groups of query heads, page sizes, windows, prompt portions
     beside single tokens. Steps of single tokens also go through the kernel that takes the new key and value from
