@@ -51,12 +51,12 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiling); prints its own line")
-    ap.add_argument("--prefill-len", type=int, default=2048, help="with --prefill-only: tokens of the prompt (the contract's point is 2,048)")
+    ap.add_argument("--prefill-len", type=int, default=2048, help="with --prefill-only: tokens of the prompt (the headline point is 2,048)")
     ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
-                    help="layer sizes of the decode workload: 7b is the contract's; xl and 20b measure the same step at the other "
+                    help="layer sizes of the decode workload: 7b is the headline's; xl and 20b measure the same step at the other "
                          "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
     ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b"],
-                    help="decode: the contract above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
+                    help="decode: the workload described above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
                          "through InferenceEngine.generate; they print their own line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -123,29 +123,41 @@ def main() -> int:
             engine.step()
         torch.cuda.synchronize()
         ctx0 = sum(s.n_cached for s in seqs) / len(seqs)
+        before = dict(engine.stats)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t = time.perf_counter()
+        ev0.record()
         for _ in range(steps):
             engine.step()
+        ev1.record()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert all(len(s.generated) >= warmup + steps and not s.done for s in seqs), "the timed steps did not all decode the whole batch"
         ctx_mean = ctx0 + (steps + 1) / 2.0
+        # the device's own clock around the same steps, and the host's share of a step: what step() takes less the time it waits
+        # for the device (src/levanter/inference/engine.py:1146-1159 logs the same split per iteration)
+        timing = {"device_ms_per_step": round(ev0.elapsed_time(ev1) / steps, 4),
+                  "host_ms_per_step": round(((engine.stats["step_s"] - before["step_s"]) - (engine.stats["wait_s"] - before["wait_s"])) / steps * 1e3, 4)}
         engine.reset()
-        return dt, ctx_mean
+        return dt, ctx_mean, timing
 
     def prefill_run(T, reps):
-        best = None
-        for rep in range(reps):
+        """One prompt of T tokens in one step, ``reps`` times after one untimed run: the median, with the fastest and slowest."""
+        times = []
+        for rep in range(reps + 1):
             engine.reset()
             engine.enqueue_requests([Request(prompt_tokens=prompts(1, T, 50 + rep)[0], request_id=rep, max_new_tokens=1)])
             torch.cuda.synchronize()
             t = time.perf_counter()
             engine.step()
             torch.cuda.synchronize()
-            d = time.perf_counter() - t
-            best = d if best is None or d < best else best
+            if rep > 0:
+                times.append(time.perf_counter() - t)
+        times.sort()
+        mid = times[len(times) // 2]
         flops = 2.0 * T * matrix_params + 2.0 * T * T * D * L + 2.0 * D * V
-        return {"value": round(T / best, 1), "tokens": T, "ms": round(best * 1e3, 3), "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
+        return {"value": round(T / mid, 1), "tokens": T, "ms": round(mid * 1e3, 3), "frac": round(flops / mid / PEAK_FLOPS[args.dtype], 4),
+                "ms_min": round(times[0] * 1e3, 3), "ms_max": round(times[-1] * 1e3, 3), "reps": reps}
 
     if args.prefill_only:
         if not 1 <= args.prefill_len < cfg.n_positions + 1:
@@ -154,7 +166,7 @@ def main() -> int:
         print(json.dumps({"prefill": prefill_run(args.prefill_len, 4), "model": f"gpt2_{args.shape} shape"}), flush=True)
         return 0
 
-    dt, ctx_mean = decode_run(args.batch, args.steps, args.warmup, seed=1)
+    dt, ctx_mean, timing = decode_run(args.batch, args.steps, args.warmup, seed=1)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     step_bytes = weight_bytes + args.batch * ctx_mean * kv_bytes_per_token
@@ -163,7 +175,7 @@ def main() -> int:
         "metric": (f"decode tok/s @ batch 8, {shape_name} shape, bf16" if args.batch == 8 and args.dtype == "bfloat16"
                    else f"decode tok/s @ batch {args.batch}, {shape_name} shape"),
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), **timing, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
         "config": {"model": f"gpt2_{args.shape} shape", "n_layer": L, "n_layer_full": full_layers, "n_embd": D, "n_head": cfg.n_head,
                    "head_dim": cfg.head_dim, "n_inner": F, "vocab_size": V, "n_positions": cfg.n_positions,
@@ -174,11 +186,18 @@ def main() -> int:
     }
     if not args.no_points:
         # prefill of one 2,048-token prompt in one step (the logits of its last token)
-        out["prefill"] = prefill_run(2048, 3)
+        out["prefill"] = prefill_run(2048, 5)
         points = {}
         for b, steps in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
-            d, _ = decode_run(b, steps, min(args.warmup, 4), seed=2 + b)
+            d, _, _ = decode_run(b, steps, min(args.warmup, 4), seed=2 + b)
             points[f"decode_b{b}"] = round(b * steps / d, 2)
+        # the same prefill with every matrix product on this repository's own kernels (none left to the vendor library)
+        kernels = engine.env.kernels
+        was, kernels.gemm_library = kernels.gemm_library, False
+        try:
+            points["prefill_own_kernels"] = prefill_run(2048, 3)["value"]
+        finally:
+            kernels.gemm_library = was
         out["points"] = points
     print(json.dumps(out), flush=True)
     return 0
@@ -193,14 +212,14 @@ def serving_workload(args) -> int:
     from levanter_amd.engine import InferenceEngine, Request
 
     ps = 16
-    if args.workload == "xl_mix":  # configs[3]: gpt2_xl sizes, 64 requests, prompts U[16, 768], 128 new tokens, portions of 256
+    if args.workload == "xl_mix":  # gpt2_xl sizes (config/gpt2_xl.yaml), 64 requests, prompts U[16, 768], 128 new tokens, portions of 256
         raw = {"model_type": "gpt2", "n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400, "vocab_size": 50257,
                "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
         n_req, new_tokens, temperature, chunk = 64, 128, 0.0, 256
         g = torch.Generator().manual_seed(3)
         lens = torch.randint(16, 769, (n_req,), generator=g).tolist()
         name = "gpt2_xl shape, 64 requests, prompts U[16,768], 128 new tokens, portions of 256"
-    else:  # configs[4]: gpt2_20b sizes, 32 requests x 1024-token prompts, 512 tokens each at temperature 1.0
+    else:  # gpt2_20b sizes (config/gpt2_20b.yaml), 32 requests x 1024-token prompts, 512 tokens each at temperature 1.0
         raw = {"model_type": "gpt2", "n_layer": 44, "n_embd": 6144, "n_head": 64, "n_inner": 24576, "vocab_size": 50257,
                "n_positions": 2048, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
         n_req, new_tokens, temperature, chunk = 32, 512, 1.0, 2048
@@ -220,7 +239,7 @@ def serving_workload(args) -> int:
     t0 = time.time()
     engine = InferenceEngine.from_config(cfg, seed=0, config=ecfg)
     torch.cuda.synchronize()
-    max_pages = engine.cache.groups[0].pool.n_pages
+    max_pages = max((g.pool.n_pages for g in engine.cache.groups), default=0)
     print(f"[bench] model ready in {time.time() - t0:.1f}s: {engine.model.weight_bytes() / 1e9:.2f} GB of weights, "
           f"{max_pages} pages of {ps} tokens", file=sys.stderr, flush=True)
 
@@ -240,6 +259,7 @@ def serving_workload(args) -> int:
     print("[bench] warm-up done, the timed run starts", file=sys.stderr, flush=True)
     seqs = engine.enqueue_requests(requests(2))
     torch.cuda.synchronize()
+    before = dict(engine.stats)
     t = time.perf_counter()
     while not all(s.done for s in seqs):
         t1 = time.perf_counter()
@@ -255,7 +275,9 @@ def serving_workload(args) -> int:
     pick = lambda q: round(step_ms[min(len(step_ms) - 1, int(q * len(step_ms)))], 3)
     out = {
         "metric": f"end-to-end generated tok/s, {name}", "value": round(generated / dt, 2), "unit": "tok/s", "n_gpus": 1,
-        "steps": len(step_ms), "warmup": 0, "ms_per_step": round(dt / len(step_ms) * 1e3, 4), "higher_is_better": True,
+        "steps": len(step_ms), "warmup": 0, "ms_per_step": round(dt / len(step_ms) * 1e3, 4),
+        "host_ms_per_step": round(((engine.stats["step_s"] - before["step_s"]) - (engine.stats["wait_s"] - before["wait_s"])) / len(step_ms) * 1e3, 4),
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
         "config": {"model": args.workload, "n_layer": cfg.n_layer, "n_layer_full": full_layers, "n_embd": cfg.n_embd, "n_head": cfg.n_head,

@@ -236,6 +236,9 @@ extern "C" int lev_linear_library(const void* a, long lda, const void* w, const 
     if (known == g_timed_index.end()) {
       if (may_time)
         g_timed_index[bucket] = time_candidates(handle, &plan, plan.candidates, a, w, residual, workspace, M, N, ldo, out_dtype, stream);
+      else
+        plan.timed = true;  // recorded into a graph with the heuristic's first kernel: eager calls of this shape keep it too,
+                            // so that a replay and an eager run of the same product give the same bits
     } else {
       // Another row count of the bucket has been timed: its kernel against the heuristic's first for this row count (a
       // kernel that won at 264 rows can lose at 320, where its tiles divide the rows differently), not all sixteen again.

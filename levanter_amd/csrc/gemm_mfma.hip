@@ -836,8 +836,17 @@ static double skinny_estimate(int M, int N, int K) {
   if (sh.row_tiles == 2) cost *= 1.2;
   return cost;
 }
+// 0: the estimate decides; 1 / 2: the skinny / the stream kernel wherever it takes the row count. For measurements of the
+// choice itself (a test times both candidates at widths the estimates were not fitted to); not used by the engine.
+static int g_force_kernel = 0;
+extern "C" int lev_linear_mfma_force(int kind) {
+  LEV_REQUIRE(kind >= 0 && kind <= 2, "linear: unknown kernel choice %d (0: by estimate, 1: skinny, 2: stream)", kind);
+  g_force_kernel = kind;
+  return 0;
+}
 static bool use_skinny(int M, int N, int K) {
   if (M > SKINNY_MAX_M) return false;
+  if (g_force_kernel) return g_force_kernel == 1;
   return skinny_estimate(M, N, K) <= 1.3 * plan_stream(M, N, K).cost;
 }
 

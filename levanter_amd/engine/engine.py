@@ -44,7 +44,10 @@ class InferenceEngine:
         self.runner = ModelRunner(model, self.cache, env, allocate=allocate)
         self.sampler = Sampler(env.kernels, env.device)
         self.scheduler = Scheduler(self.cache, config, self.runner.max_len)
-        self.stats = {"steps": 0, "commits": 0, "tokens_in": 0, "launch_s": 0.0}
+        # launch_s: the host's time to plan tables and launch kernels; wait_s: the time it then waited for the device (the copy
+        # of the sampled tokens); step_s: all of step(). The host's own share of a step is step_s - wait_s, as the reference
+        # logs it per iteration (src/levanter/inference/engine.py:1146-1159: host = total - device wait).
+        self.stats = {"steps": 0, "commits": 0, "tokens_in": 0, "launch_s": 0.0, "wait_s": 0.0, "step_s": 0.0}
         self._pending: Optional[_Launched] = None  # a step launched ahead of the one being committed
 
     # ---- construction -------------------------------------------------------------------------
@@ -118,6 +121,19 @@ class InferenceEngine:
         for the host between steps. What cannot be known without the tokens (a stop sequence that ends a request) is
         settled afterwards: the request's row of the step launched ahead is ignored, and what that row wrote lies in
         pages that its request no longer owns and nobody reads."""
+        t_step = time.perf_counter()
+        try:
+            return self._step()
+        finally:
+            self.stats["step_s"] += time.perf_counter() - t_step
+
+    def _read(self, sample):
+        t0 = time.perf_counter()
+        out = self.sampler.read(sample)
+        self.stats["wait_s"] += time.perf_counter() - t0
+        return out
+
+    def _step(self) -> List[Sequence_]:
         pend = self._pending
         self._pending = None
         if pend is None:
@@ -131,7 +147,7 @@ class InferenceEngine:
             ahead = self.scheduler.plan_lookahead(pend.plan)
             if ahead is not None:
                 nxt = self._launch(ahead[0], (pend.sample.tokens, ahead[1]) if ahead[1] else None)
-        toks, lps = ([], []) if pend.sample is None else self.sampler.read(pend.sample)
+        toks, lps = ([], []) if pend.sample is None else self._read(pend.sample)
         finished = self.scheduler.commit(pend.plan, toks, lps)
         if nxt is not None:
             if all(e.seq.done for e in nxt.plan):  # every request of the step launched ahead has ended meanwhile

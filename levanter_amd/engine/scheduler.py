@@ -142,7 +142,8 @@ class Scheduler:
             # pages ran out: preempt the youngest running sequence, or fail the only one
             victim = max(self.running, key=lambda s: s.order)
             if len(self.running) == 1:
-                self._finish(victim, f"error: out of pages (needs more than the pool of {self.cache.groups[0].pool.n_pages} pages)")
+                pools = ", ".join(str(g.pool.n_pages) for g in self.cache.groups) or "none"
+                self._finish(victim, f"error: out of pages (needs more than the pool holds: {pools} pages)")
                 if not self.waiting:
                     return []
                 continue

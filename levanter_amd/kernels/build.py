@@ -270,6 +270,7 @@ register_unit("gemm_mfma", ["gemm_mfma.hip"], signatures={
     "lev_linear_mfma": [_P, _L, _P, _P, _P, _L, _P, _L, _P] + [_I] * 6 + [_P],
     "lev_linear_mfma_workspace": [_I, _I, _I],
     "lev_linear_mfma_ranges": [_I, _I, _I],
+    "lev_linear_mfma_force": [_I],
     "lev_linear_mfma_finish": [_P, _P, _P, _L, _P, _L] + [_I] * 5 + [_P],
 })
 # the vendor library's GEMM (hipBLASLt) behind the same interface

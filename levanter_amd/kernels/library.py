@@ -224,7 +224,7 @@ class HipKernels:
         with it. A buffer that is outgrown stays alive, because recorded HIP graphs may point at it; while a graph is
         being recorded a buffer that is too small is not replaced but a fresh one handed out, which stays with the graph."""
         last = self._ws_last
-        if last is not None and last[0] is device and last[2] >= need:
+        if last is not None and last[0] == device and last[2] >= need:
             return last[1]
         ws = self._ws.get(device)
         if ws is not None and ws.numel() >= need:

@@ -11,7 +11,10 @@ from typing import Dict
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description="feed token ids through a model step by step, write logits")
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", help="folder with config.json and model.safetensors")
+    ap.add_argument("--random-config", help="instead of --model: a config.json (a file, or the JSON itself) whose model gets random weights "
+                                            "drawn from --seed, the same as a folder written from that configuration and seed holds")
+    ap.add_argument("--seed", type=int, default=0, help="with --random-config: the seed of the weights")
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
@@ -19,6 +22,8 @@ def main(argv=None) -> int:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--max-seqs", type=int, default=8)
     args = ap.parse_args(argv)
+    if (args.model is None) == (args.random_config is None):
+        ap.error("give either --model or --random-config")
 
     print("trace_run: loading torch and the HIP library ...", file=sys.stderr, flush=True)
     import torch  # noqa: F401
@@ -29,7 +34,21 @@ def main(argv=None) -> int:
     from levanter_amd.engine.loading import load_model, make_cache, make_env
 
     env = make_env(args.dtype)
-    config, model = load_model(args.model, env)
+    if args.model is not None:
+        config, model = load_model(args.model, env)
+    else:
+        from levanter_amd.config import LmConfig
+        from levanter_amd.parts import DecoderLm
+        from levanter_amd.weights import random_tensors
+
+        raw = args.random_config
+        if not raw.lstrip().startswith("{"):
+            with open(raw, encoding="utf-8") as f:
+                raw = f.read()
+        config = LmConfig.from_dict(json.loads(raw))
+        spec = config.model_spec()
+        # drawn on the CPU, stored in the compute dtype: tensor for tensor what write_random_model puts into a folder
+        model = DecoderLm(spec, random_tensors(spec, args.seed, dtype=env.dtype, device="cpu"), env)
     ps = args.page_size
     n_pages = max(1, (args.max_tokens + ps - 1) // ps)
     if 64 % ps != 0 and ps % 64 != 0:  # counts are rounded to 64, pages are not: every live request may need one page more

@@ -86,3 +86,31 @@ def check_all_cuttings(label, raw, seed, dtype, lengths, page_size=16):
             clear = (top2[:, 0] - top2[:, 1]) > 2e-2
             assert bool((got.argmax(-1)[clear] == w.argmax(-1)[clear]).all())
             assert float((torch.softmax(got.double(), -1) - torch.softmax(w, -1)).abs().max()) < 1e-2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_from_a_configuration_and_a_seed(dtype):
+    """``--random-config`` with ``--seed`` in place of ``--model``: the weights are those a folder written from the same
+    configuration and seed holds, so the logits are the same bits."""
+    import json
+
+    raw, seed = TINY["A"]
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    d = write_model(raw, seed, store)
+    reqs = TR.random_requests(raw["vocab_size"], [40, 21], 3)
+    steps = TR.number(TR.trace_portions(reqs))
+    out_folder = run_trace(d, dtype, steps, 128)
+    out = tempfile.mkdtemp(prefix="lev_trace_")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--random-config", json.dumps(raw), "--seed", str(seed), "--dtype", dtype,
+           "--out", out, "--max-tokens", "128"]
+    p = subprocess.run(cmd, input=TR.to_jsonl(steps), capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-3000:]
+    n = 0
+    for s_ in steps:
+        f = os.path.join(out_folder, f"{s_['step']}.f32")
+        if os.path.exists(f):
+            assert torch.equal(read_step(out, s_["step"], raw["vocab_size"]), read_step(out_folder, s_["step"], raw["vocab_size"]))
+            n += 1
+    assert n > 0
+    p = subprocess.run(cmd[:2] + ["--dtype", dtype, "--out", out, "--max-tokens", "64"], input="", capture_output=True, text=True, timeout=120)
+    assert p.returncode != 0 and "either --model or --random-config" in p.stderr
