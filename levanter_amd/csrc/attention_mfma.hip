@@ -231,6 +231,7 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
                                              const int* __restrict__ block_tables, int bt_stride, int t0, int rows, int h,
                                              int H, int KVH, int ps_shift, float scale, int window, float softcap,
                                              const float* __restrict__ score_bias, int bias_len, KsPtr Ks, VsPtr Vs) {
+  if (rows <= 0) return;  // an empty tile (a step filled up to a fixed number of tiles): nothing to do, for the whole workgroup
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int fr = lane & 15, g = lane >> 4;
   const int kvh = h / (H / KVH);

@@ -238,11 +238,15 @@ class InferenceEngine:
         # of anything (the library keeps the kernel it timed fastest for row counts up to the same multiple of 64; timing
         # takes a fifth of a second at 20B sizes)
         rounds = self.config.max_rounds  # decode steps that may pass before a waiting request is admitted
-        for d in range(1, most, 64):
-            self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=rounds + 4) for i in range(d)])
+        from .step import MIXED_DECODE_BUCKET
+
+        # one run for every number of single tokens that such steps are filled up to, with prompt tokens for two full steps:
+        # a shape that has come twice is recorded and replayed from then on
+        for d in sorted({min(d, most - 1) for d in range(1, most, MIXED_DECODE_BUCKET)}):
+            self.enqueue_requests([Request(prompt_tokens=[(3 * i + 1) % v], request_id=-1 - i, max_new_tokens=rounds + 8) for i in range(d)])
             self.step()
-            self.enqueue_requests(prompts(min(limit, one * max(1, min(most - d, self.config.max_seqs_in_prefill))), -1 - d))
-            for _ in range(rounds + 8):
+            self.enqueue_requests(prompts(min(2 * limit, one * max(1, min(most - d, self.config.max_seqs_in_prefill))), -1 - d))
+            for _ in range(rounds + 12):
                 if self.scheduler.idle and self._pending is None:
                     break
                 self.step()

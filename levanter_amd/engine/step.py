@@ -112,8 +112,9 @@ class ModelRunner:
                 self.cache.extend(e.handle, len(e.tokens))
                 extended.append(e)
             graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
-            batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable)
-            if graphable:
+            mixed = self._mixed_step_shape(entries) if self.use_graphs and not graphable else None
+            batch = self._build_host(entries, pad_blocks=GRAPH_BLOCK_BUCKET if graphable else 1, pad_batch=graphable, mixed=mixed)
+            if graphable or mixed is not None:
                 logits = self._run_graphed(batch, token_feed)[:batch.n_rows_real]
                 if copy_out:
                     logits = logits.clone()
@@ -130,7 +131,29 @@ class ModelRunner:
         return logits
 
     # ------------------------------------------------------------------------------------
-    def _build_host(self, entries: Sequence[StepEntry], pad_blocks: int = 1, pad_batch: bool = False) -> "HostBatch":
+    def _mixed_step_shape(self, entries: Sequence[StepEntry]) -> Optional["MixedShape"]:
+        """The shape that a step of prompt portions beside single tokens is filled up to, so that serving meets a handful
+        of such shapes and can replay them as graphs: the single tokens to a multiple of ``MIXED_DECODE_BUCKET`` (with
+        ghosts, as in steps of single tokens), room for up to ``MIXED_MAX_PORTIONS`` portions (request rows, wanted rows
+        and the partial attention tiles they may add: empty tiles fill the rest), block tables at their full width. The
+        portions' token count stays exact: a scheduler fills its budget, so most steps of a busy engine have the same.
+        None: this step has more portions or more wanted rows than the shape holds, or so many tokens that the host's
+        launches are a small part of it (a recorded graph keeps its activations for as long as it lives), and runs as it is."""
+        portions = [len(e.tokens) for e in entries if len(e.tokens) > 1]
+        if not 1 <= len(portions) <= MIXED_MAX_PORTIONS:
+            return None
+        singles = len(entries) - len(portions)
+        n_decode = -(-singles // MIXED_DECODE_BUCKET) * MIXED_DECODE_BUCKET
+        if sum(portions) + n_decode > MIXED_GRAPH_MAX_TOKENS:
+            return None
+        shape = MixedShape(n_decode=n_decode, n_seqs=n_decode + MIXED_MAX_PORTIONS, n_rows=n_decode + MIXED_MAX_PORTIONS,
+                           n_tiles=sum(portions) // self.prefill_tile_rows + MIXED_MAX_PORTIONS)
+        if sum(len(e.want) for e in entries) > shape.n_rows:
+            return None
+        return shape
+
+    def _build_host(self, entries: Sequence[StepEntry], pad_blocks: int = 1, pad_batch: bool = False,
+                    mixed: Optional["MixedShape"] = None) -> "HostBatch":
         """Everything the GPU needs to know about the step, in one int32 buffer with a layout that
         depends only on (tokens, requests, wanted rows, tiles, single tokens, blocks per request).
 
@@ -180,6 +203,21 @@ class ModelRunner:
                 rows.extend(range(T, T + ghosts))  # a ghost's logits are its own row's: no row is wanted twice
                 S += ghosts
                 T += ghosts
+        if mixed is not None:
+            ghosts = mixed.n_decode - len(decode)
+            if ghosts > 0:  # ghost tokens as above, each with a request row of its own (a copy of the first request's)
+                tokens = np.concatenate([tokens, np.zeros(ghosts, np.int32)])
+                positions = np.concatenate([positions, np.zeros(ghosts, np.int32)])
+                token_seq = np.concatenate([token_seq, np.arange(S, S + ghosts, dtype=np.int32)])
+                decode.extend(range(T, T + ghosts))
+                S += ghosts
+                T += ghosts
+            seq_slots = np.concatenate([seq_slots, np.full(mixed.n_seqs - len(seq_slots), seq_slots[0], np.int32)])  # rows no token names
+            S = mixed.n_seqs
+            # wanted rows nobody reads: a ghost's own row where there is one (the norm before the head takes a row twice)
+            rows.extend([n_real_tokens + i % ghosts if ghosts > 0 else 0 for i in range(mixed.n_rows - len(rows))])
+            tile_list.extend([(0, 0, 0)] * (mixed.n_tiles - len(tile_list)))  # empty tiles: their workgroups return at once
+            max_blocks = cache.max_pages_per_seq
         # the attention kernel pairs tile i with tile n - 1 - i: sorted by falling key range, pairs have equal work
         tile_list.sort(key=lambda x: -x[0])
         tiles: List[int] = [v for _, first, nr in tile_list for v in (first, nr)]
@@ -246,10 +284,11 @@ class ModelRunner:
         self.env.kernels.feed_tokens(dev[b.offs[0]:b.offs[0] + n], device_tokens, rows, n)
 
     def _run_graphed(self, b: "HostBatch", token_feed=None) -> torch.Tensor:
-        """A step of single tokens has a kernel sequence that depends only on (requests, wanted rows,
-        blocks per request): the second time such a step comes it is captured into a HIP graph whose
-        inputs live in a fixed device buffer; later steps copy their tables there and replay it."""
-        key = (b.n_seqs, b.n_rows, b.max_blocks)
+        """A step's kernel sequence depends only on its counts (tokens, requests, wanted rows, attention tiles, single
+        tokens, blocks per request), which steps of single tokens and mixed steps are filled up to a few values of: the
+        second time such a step comes it is captured into a HIP graph whose inputs live in a fixed device buffer; later
+        steps copy their tables there and replay it."""
+        key = (b.n_tokens, b.n_seqs, b.n_rows, b.n_tiles, b.n_decode, b.max_blocks)
         entry = self._graphs.get(key)
         if entry is None:  # first time: run eagerly (also loads every kernel the graph will need)
             self._graphs[key] = "seen"
@@ -281,6 +320,10 @@ class ModelRunner:
         return entry.logits
 
 
+MIXED_DECODE_BUCKET = 16  # single tokens beside prompt portions are filled up to a multiple of this
+MIXED_MAX_PORTIONS = 4    # prompt portions a replayable mixed step has room for
+MIXED_GRAPH_MAX_TOKENS = 512  # larger mixed steps are not recorded: the GPU's time dwarfs the host's, and a graph holds its activations
+
 N_FIXED = 8  # arrays of the step's buffer ahead of the cache groups' (block tables, destinations)
 GRAPH_BLOCK_BUCKET = 16  # block tables of graphed steps are padded to a multiple of this many pages
 MAX_GRAPHS = 48
@@ -290,6 +333,16 @@ def graph_batch_bucket(n: int) -> int:
     """Batch size that a graphed step of ``n`` single tokens is filled up to: small batches stay as they are,
     larger ones go to the next multiple of 8 (the GEMM kernels work on row tiles of 16 anyway)."""
     return n if n <= 4 else (n + 7) // 8 * 8
+
+
+@dataclass(frozen=True)
+class MixedShape:
+    """Counts that a step of prompt portions beside single tokens is filled up to (see ``_mixed_step_shape``)."""
+
+    n_decode: int
+    n_seqs: int
+    n_rows: int
+    n_tiles: int
 
 
 @dataclass

@@ -768,6 +768,75 @@ def test_decode_steps_replayed_from_a_hip_graph_equal_eager_steps(dtype, monkeyp
     assert all(r.cache.groups[0].pool.n_free < 40 for r, _ in runners)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_steps_are_filled_up_to_a_few_shapes_and_replayed_from_graphs(dtype, monkeypatch):
+    """Steps of prompt portions beside single tokens are filled up (ghost single tokens to a multiple of 16, room for four
+    portions, empty attention tiles, full-width block tables) so that steps with the same number of prompt tokens share a
+    shape and are replayed from a HIP graph from their second occurrence on. Every such step equals the same step run
+    eagerly without any filling (32-bit: bit for bit), with one to three portions, requests that end, a step whose many
+    wanted rows do not fit the shape (it runs as it is), and the caches agree afterwards."""
+    from levanter_amd.config import InferenceEngineConfig
+    from levanter_amd.engine import ModelRunner, StepEntry
+    from levanter_amd.engine.loading import load_model, make_cache
+    import levanter_amd.engine.step as step_mod
+
+    monkeypatch.setattr(step_mod, "MIXED_DECODE_BUCKET", 4)
+    d = write_model(TINY_A, 0, torch.float32 if dtype == "float32" else torch.bfloat16)
+    env = _env(dtype)
+    _, model = load_model(d, env)
+    cfg = InferenceEngineConfig(max_pages=120, max_seqs=16, page_size=16, max_pages_per_seq=8, compute_dtype=dtype)
+    runners = []
+    for graphs in (True, False):
+        cache = make_cache(model, cfg)
+        runners.append((ModelRunner(model, cache, env, use_graphs=graphs), cache))
+    g = torch.Generator().manual_seed(21)
+    names = [f"r{i}" for i in range(14)]
+    toks = {k: torch.randint(0, 512, (120,), generator=g).tolist() for k in names}
+    handles = [{k: c.open(k) for k in names[:6]} for _, c in runners]
+    for (r, _), h in zip(runners, handles):  # six requests that decode from now on
+        r.step([StepEntry(h[k], toks[k][:2 + 3 * i], []) for i, k in enumerate(names[:6])])
+    live = list(names[:6])
+    tol = dict(rtol=0, atol=0) if dtype == "float32" else dict(rtol=2e-2, atol=8e-3)
+    # 40 prompt tokens a step, cut into one to three portions of newcomers; the single tokens go 6, 6, 5 (one ends), ...
+    plans = [[("r6", 40)], [("r6", 30), ("r7", 10)], [("r7", 25), ("r8", 13), ("r9", 2)], [("r8", 40)], [("r9", 38), ("r10", 2)],
+             [("r10", 40)], [("r10", 20), ("r11", 20)], [("r11", 40)], [("r12", 40)], [("r12", 33), ("r13", 7)]]
+    replays = 0
+    for i, plan in enumerate(plans):
+        if i in (2, 6):
+            gone = live.pop(1)
+            for (_, c), h in zip(runners, handles):
+                c.close(h.pop(gone))
+        outs = []
+        for (r, c), h in zip(runners, handles):
+            entries = [StepEntry(h[k], [toks[k][h[k].length]], [0]) for k in live]
+            for k, n in plan:
+                if k not in h:
+                    h[k] = c.open(k)
+                entries.append(StepEntry(h[k], toks[k][h[k].length:h[k].length + n], [n - 1]))
+            before = sum(1 for v in r._graphs.values() if v != "seen")
+            outs.append(r.step(entries).cpu())
+            c.check_invariants()
+        assert outs[0].shape == (len(live) + len(plan), 512)
+        torch.testing.assert_close(outs[0], outs[1], **tol, msg=lambda m: f"mixed step {i}: {m}")
+    graphs = {k: v for k, v in runners[0][0]._graphs.items() if v != "seen"}
+    # single tokens 6 and 5 fill up to 8, 4 stays 4: two shapes of 40 prompt tokens, both recorded and replayed
+    assert len(graphs) == 2 and all(k[0] - k[4] == 40 and k[4] in (4, 8) for k in graphs), list(graphs)
+    # a step that wants every row of its portion does not fit the shape's wanted rows: it runs as it is, and is right
+    outs = []
+    for (r, c), h in zip(runners, handles):
+        k = "r13"
+        n = 30
+        outs.append(r.step([StepEntry(h[x], [toks[x][h[x].length]], [0]) for x in live]
+                           + [StepEntry(h[k], toks[k][h[k].length:h[k].length + n], list(range(n)))]).cpu())
+    assert outs[0].shape == (len(live) + 30, 512)
+    torch.testing.assert_close(outs[0], outs[1], **tol)
+    # what the steps wrote is the same with and without filling: every live request reads all of its cache once more
+    last = []
+    for (r, _), h in zip(runners, handles):
+        last.append(r.step([StepEntry(h[k], toks[k][h[k].length:h[k].length + 3], [2]) for k in sorted(h)]).cpu())
+    torch.testing.assert_close(last[0], last[1], **tol)
+
+
 def test_more_step_shapes_than_graphs_are_kept(monkeypatch):
     """At most ``MAX_GRAPHS`` shapes are remembered; one more and every recorded graph is dropped (its shape is recorded
     again when it comes twice more). With room for 3 and a block-table width that changes every 16 tokens, 110 decode
