@@ -144,7 +144,8 @@ class ModelRunner:
             return None
         singles = len(entries) - len(portions)
         n_decode = -(-singles // MIXED_DECODE_BUCKET) * MIXED_DECODE_BUCKET
-        if sum(portions) + n_decode > MIXED_GRAPH_MAX_TOKENS:
+        # the GPU's time for a step grows with tokens x width^2, the host's with the number of launches alone
+        if (sum(portions) + n_decode) * self.model.dim ** 2 > MIXED_GRAPH_MAX_WORK:
             return None
         shape = MixedShape(n_decode=n_decode, n_seqs=n_decode + MIXED_MAX_PORTIONS, n_rows=n_decode + MIXED_MAX_PORTIONS,
                            n_tiles=sum(portions) // self.prefill_tile_rows + MIXED_MAX_PORTIONS)
@@ -322,7 +323,9 @@ class ModelRunner:
 
 MIXED_DECODE_BUCKET = 16  # single tokens beside prompt portions are filled up to a multiple of this
 MIXED_MAX_PORTIONS = 4    # prompt portions a replayable mixed step has room for
-MIXED_GRAPH_MAX_TOKENS = 512  # larger mixed steps are not recorded: the GPU's time dwarfs the host's, and a graph holds its activations
+# Larger mixed steps are not recorded: the GPU's time dwarfs the host's, and a graph holds its activations. In tokens x width^2:
+# 512 tokens of a 4,096-wide model (a GPT-2 XL step of any size, 227 tokens at 6,144 wide).
+MIXED_GRAPH_MAX_WORK = 512 * 4096 ** 2
 
 N_FIXED = 8  # arrays of the step's buffer ahead of the cache groups' (block tables, destinations)
 GRAPH_BLOCK_BUCKET = 16  # block tables of graphed steps are padded to a multiple of this many pages
