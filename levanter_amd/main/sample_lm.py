@@ -8,7 +8,8 @@ Options carry the names and meanings of the reference's ``SampleLmConfig``
 and model.safetensors), ``tokenizer``, ``engine`` (``InferenceEngineConfig``), ``prompts``,
 ``stop_sequence``, ``max_new_tokens`` (192), ``temperature`` (0.7), ``seed`` (2), ``n_generations`` (1),
 ``n_rounds`` (4; the same batch is generated that many times, the first round includes set-up),
-``profile``. ``trainer.mp`` keeps the reference's precision string ("p=bfloat16,c=bfloat16"); its compute
+``profile`` (the reference starts its profiler from the second round on, sample_lm.py:137-152; here every round then prints
+how its time divides into the host's own work, the launches among it, and waiting for the GPU). ``trainer.mp`` keeps the reference's precision string ("p=bfloat16,c=bfloat16"); its compute
 part sets ``engine.compute_dtype``. Added: ``prompt_ids`` and ``stop_ids`` give token ids directly, so that
 no tokenizer is needed; ``random_config`` / ``random_seed`` run a randomly initialised model of a
 configuration instead of a checkpoint.
@@ -131,10 +132,17 @@ def main(config: SampleLmConfig) -> int:
                                                         temperature=config.temperature, key=fold_in(base_key, ridx)),
                         n_generations=config.n_generations)
                 for ridx, toks in enumerate(prompt_ids)]
+        before = dict(engine.stats)
         result = engine.generate(reqs)
         dt = time.time() - time_in
         print(f"round {r}: {result.total_generated} tokens in {len(result.tokens)} sequences, {dt:.2f} s "
               f"({result.total_generated / max(dt, 1e-9):.1f} tok/s)", flush=True)
+        if config.profile:
+            d = {k: engine.stats[k] - before[k] for k in before}
+            n = max(1, d["commits"])
+            print(f"round {r} profile: {d['steps']} steps of {d['tokens_in']} tokens in all; a step took the host {1e3 * (d['step_s'] - d['wait_s']) / n:.3f} ms "
+                  f"({1e3 * d['launch_s'] / n:.3f} ms of it planning tables and launching kernels) and {1e3 * d['wait_s'] / n:.3f} ms of waiting for the GPU",
+                  flush=True)
         for seq_id, out in enumerate(result.tokens):
             print(f"round {r} sequence {seq_id} ({len(out)} tokens, {result.finish_reasons[seq_id]}): {out}")
             if tokenizer is not None:

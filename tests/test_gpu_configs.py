@@ -191,8 +191,10 @@ def test_command_line_from_a_folder_to_greedy_tokens():
     g = torch.Generator().manual_seed(4)
     prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (9, 40, 1)]
     rounds, out = _sample_lm(["--hf_checkpoint", d, "--prompt_ids", json.dumps(prompts), "--temperature", "0", "--max_new_tokens", "16",
-                              "--n_rounds", "2", "--trainer.mp", "p=f32,c=f32", "--engine.max_seqs", "4", "--engine.max_pages_per_seq", "8"])
+                              "--n_rounds", "2", "--trainer.mp", "p=f32,c=f32", "--engine.max_seqs", "4", "--engine.max_pages_per_seq", "8",
+                              "--profile", "true"])
     assert sorted(rounds) == [0, 1] and "float32" in out
+    assert out.count(" profile: ") == 2 and "waiting for the GPU" in out  # one line a round on where its time went
     for r in rounds.values():
         assert sorted(r) == [0, 1, 2]
         for i, p in enumerate(prompts):
