@@ -250,3 +250,34 @@ def test_command_line_sampling_equals_the_python_entry_point():
                            for i, p in enumerate(prompts)])
     assert [rounds[0][i][0] for i in range(4)] == res.tokens
     assert len({tuple(t) for t in res.tokens}) == 4  # generations of one request differ: it is sampling
+
+
+def test_command_line_with_text_prompts_and_a_tokenizer_file():
+    """Prompts and the stop sequence as text, as the reference's command takes them (src/levanter/main/sample_lm.py:97-121:
+    the tokenizer encodes each prompt and the stop sequence without special tokens): a word-level ``tokenizer.json`` in the
+    model folder. The ids are the tokenizer's, the tokens the plain implementation's greedy continuation up to the stop word,
+    and the text lines are the tokenizer's decoding of them."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    d = write_model(TINY_A, 0, torch.float32)
+    w = read_weights(d)
+    vocab = {f"w{i}": i for i in range(TINY_A["vocab_size"])}
+    tok = Tokenizer(models.WordLevel(vocab=vocab, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.save(os.path.join(d, "tokenizer.json"))
+    texts = ["w5 w17 w3 w400", "w77"]
+    ids = [[5, 17, 3, 400], [77]]
+    whole = [P.plain_greedy_generate(w, TINY_A, p, 12) for p in ids]
+    stop_word = f"w{whole[0][4]}"  # the fifth generated token of prompt 0 ends it (or an earlier occurrence of the same word)
+    expect = []
+    for p, g in zip(ids, whole):
+        n = next((n for n in range(1, len(g) + 1) if P.plain_is_stop(p + g[:n], [[whole[0][4]]])), len(g))
+        expect.append(g[:n])
+    rounds, out = _sample_lm(["--hf_checkpoint", d, "--prompts", json.dumps(texts), "--stop_sequence", stop_word, "--temperature", "0",
+                              "--max_new_tokens", "12", "--n_rounds", "1", "--trainer.mp", "p=f32,c=f32", "--engine.max_pages_per_seq", "8"])
+    for i, p in enumerate(ids):
+        assert f"prompt {i} ({len(p)} tokens): {p}" in out
+        toks, reason = rounds[0][i]
+        assert toks == expect[i] and reason == ("stop" if P.plain_is_stop(p + toks, [[whole[0][4]]]) else "length")
+        assert f"round 0 sequence {i} text: {' '.join(f'w{t}' for t in toks)}" in out
+    assert rounds[0][0][1] == "stop" and len(rounds[0][0][0]) <= 5
