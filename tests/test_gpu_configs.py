@@ -52,6 +52,51 @@ def test_a_head_size_of_40_runs_in_32_bit_and_is_refused_in_bfloat16():
     assert p.returncode != 0 and "head_dim=40 must be a multiple of 16" in p.stderr
 
 
+@pytest.mark.parametrize("seed", [1, 7])
+def test_configurations_drawn_at_random(seed):
+    """Four configurations a seed, every size and option drawn at random: one to twelve heads of 16 to 128 dimensions in
+    steps of 16 (in 32-bit also 8, 24, 40, 56 and 72), one to three layers, an inner width that is any multiple of 8 or
+    left to the default, a vocabulary and a position table of any size, each of the reference's activation names
+    (src/levanter/utils/activation.py:18-40), three values of eps, the 1/(layer + 1) factor and the biases on or off; the
+    four cuttings through ``bin/trace_run``. 32-bit is held to the tolerance of the other replay tests. bfloat16 is
+    compared with the plain implementation rounded at the same places, relative to the size of the logits as at the 7B
+    widths: wider models have larger logits and rounding differences that grow with them (a step's r.m.s. error within
+    1.5e-2 of the logits' r.m.s., its largest within 8 times that)."""
+    import random
+
+    rng = random.Random(seed)
+    acts = ["relu", "silu", "swish", "gelu", "gelu_new", "quick_gelu", "tanh"]
+    for ci in range(4):
+        dtype = "float32" if ci % 2 == 0 else "bfloat16"
+        hd = rng.choice([16, 32, 48, 64, 80, 96, 112, 128]) if dtype == "bfloat16" else rng.choice([8, 24, 40, 16, 56, 72, 128])
+        nh = rng.choice([1, 2, 3, 5, 7, 12])
+        raw = dict(model_type="gpt2", n_layer=rng.choice([1, 2, 3]), n_embd=hd * nh, n_head=nh,
+                   n_inner=rng.choice([None, 8 * rng.randrange(3, 300)]), vocab_size=rng.randrange(300, 6000),
+                   n_positions=rng.randrange(70, 330), layer_norm_epsilon=rng.choice([1e-5, 1e-6, 3e-4]),
+                   activation_function=rng.choice(acts), scale_attn_by_inverse_layer_idx=rng.random() < 0.5, use_bias=rng.random() < 0.8)
+        what = f"seed {seed} configuration {ci} {dtype} {json.dumps(raw)}"
+        print(what, flush=True)
+        d = write_model(raw, 5 + ci, torch.float32 if dtype == "float32" else torch.bfloat16)
+        weights = read_weights(d)
+        n_pos = raw["n_positions"]
+        reqs = TR.random_requests(raw["vocab_size"], [min(n_pos, n) for n in (rng.randrange(40, 130), 45, n_pos, rng.randrange(33, 70), 64, 33)],
+                                  21 + ci)
+        rounding = P.bf16_rounding if dtype == "bfloat16" else (lambda x: x)
+        plain = {rid: P.plain_logits(weights, raw, torch.tensor(t), rounding=rounding) for rid, t in reqs.items()}
+        steps = TR.number(TR.trace_whole(reqs) + TR.trace_prefill_then_singles(reqs) + TR.trace_portions(reqs)
+                          + TR.trace_mixed(reqs, seed=3 + ci))
+        out = run_trace(d, dtype, steps, TR.peak_tokens(steps))
+        want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+        rms = float(torch.cat([w.flatten() for w in plain.values()]).pow(2).mean().sqrt())
+        for k, w in want.items():
+            got = read_step(out, k, raw["vocab_size"]).double()
+            if dtype == "float32":
+                torch.testing.assert_close(got, w, **TOL_F32, msg=lambda m: f"{what} step {k}: {m}")
+            else:
+                err = (got - w).abs()
+                assert float(err.pow(2).mean().sqrt()) <= 1.5e-2 * rms and float(err.max()) <= 8 * 1.5e-2 * rms, (what, k, float(err.max()), rms)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_reference_s_schedules_through_trace_run(dtype):
     """The step schedules of the reference's paged-attention tests (tests/inference/test_paged_attention.py:293-442):
