@@ -638,6 +638,62 @@ def test_a_window_whose_first_block_has_lost_its_leading_pages(K, dtype, H, KVH,
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pools_of_more_than_two_to_the_31_elements(K, dtype):
+    """A key pool and a value pool of 2^31 + 2^20 elements each (what a cache sized from free memory holds for a small
+    model): requests whose pages lie at the pools' far end, where an element offset no longer fits 32 bits. Written by
+    the KV-write kernel and by the decode kernel that writes the new key itself, read by prompt portions and single
+    tokens; compared with the plain statement over a copy of just those pages."""
+    H, KVH, HD, PS = 16, 8, 128, 16
+    elems = KVH * HD * PS
+    n_pages = (1 << 31) // elems + 64
+    assert n_pages * elems > (1 << 31)
+    runs = [(1, 300), (70, 150), (1, 17), (130, 130)]
+    kv_lens = [k for _, k in runs]
+    need = sum((k + PS - 1) // PS for k in kv_lens)
+    far = n_pages - need - 5
+    small = random_block_tables(kv_lens, PS, need + 5, 4, "cpu")       # pages 0 .. need + 4 of a small pool
+    bt = torch.where(small >= 0, small + far, small)                    # the same pages at the far end of the large one
+    kd = torch.full((n_pages, elems), float("nan"), dtype=dtype, device=DEV)
+    vd = torch.full((n_pages, elems), float("nan"), dtype=dtype, device=DEV)
+    kp = torch.full((need + 5, elems), float("nan"), dtype=dtype)
+    vp = torch.full((need + 5, elems), float("nan"), dtype=dtype)
+    for s_, n in enumerate(kv_lens):
+        k, v = _rand(n, KVH * HD, dtype=dtype, seed=300 + s_), _rand(n, KVH * HD, dtype=dtype, seed=350 + s_)
+        EMU.kv_write(k, v, kp, vp, torch.tensor(dest_for(small, s_, range(n), PS), dtype=torch.int32), KVH, HD, PS)
+        upto = n - 1 if runs[s_][0] == 1 else n  # the single tokens' own keys are written by the attention kernel below
+        K.kv_write(k[:upto].to(DEV), v[:upto].to(DEV), kd, vd, torch.tensor(dest_for(bt, s_, range(upto), PS), dtype=torch.int32, device=DEV),
+                   KVH, HD, PS)
+    T = sum(q for q, _ in runs)
+    q = _rand(T, H * HD, dtype=dtype, seed=11)
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=1 / math.sqrt(HD) / 2, window=None)
+    want = torch.empty(T, H * HD, dtype=dtype)
+    EMU.paged_attention(q, want, kp, vp, make_meta(runs, "cpu"), block_tables=small, **args)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    # the single tokens first, as a decode step that brings their keys and values along; then all four runs together
+    singles = [i for i, (qn, _) in enumerate(runs) if qn == 1]
+    first_row = [sum(qn for qn, _ in runs[:i]) for i in range(len(runs))]
+    k_new = torch.stack([_rand(kv_lens[i], KVH * HD, dtype=dtype, seed=300 + i)[-1] for i in singles]).to(DEV)
+    v_new = torch.stack([_rand(kv_lens[i], KVH * HD, dtype=dtype, seed=350 + i)[-1] for i in singles]).to(DEV)
+    dest = torch.tensor([dest_for(bt, i, [kv_lens[i] - 1], PS)[0] for i in singles], dtype=torch.int32, device=DEV)
+    got1 = torch.full((len(singles), H * HD), float("nan"), dtype=dtype, device=DEV)
+    fused = K.paged_attention(q[[first_row[i] for i in singles]].to(DEV), got1, kd, vd, make_meta([runs[i] for i in singles], DEV), k_new=k_new,
+                              v_new=v_new, dest=dest, block_tables=bt[singles].to(DEV), **args)
+    if not fused:  # this dtype has no kernel that writes the new key itself: write it, then attend
+        K.kv_write(k_new, v_new, kd, vd, dest, KVH, HD, PS)
+        K.paged_attention(q[[first_row[i] for i in singles]].to(DEV), got1, kd, vd, make_meta([runs[i] for i in singles], DEV),
+                          block_tables=bt[singles].to(DEV), **args)
+    torch.testing.assert_close(got1.cpu().float(), want[[first_row[i] for i in singles]].float(), **tol)
+    used = torch.arange(far, far + need + 5, device=DEV)
+    torch.testing.assert_close(kd[used].cpu(), kp, rtol=0, atol=0, equal_nan=True)
+    torch.testing.assert_close(vd[used].cpu(), vp, rtol=0, atol=0, equal_nan=True)
+    got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q.to(DEV), got, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    del kd, vd
+    torch.cuda.empty_cache()
+
+
 def test_paged_attention_random_cases(K):
     """Forty random cases in bfloat16: head sizes 16 .. 128, groups of query heads, page sizes, windows, prompt portions
     beside single tokens. Steps of single tokens also go through the kernel that takes the new key and value from
