@@ -13,7 +13,7 @@
 //
 // Page layouts (elements): keys [page][kv_head][HD/8][PS][8], values [page][kv_head][HD][PS].
 //
-//   prefill kernel: one workgroup (4 waves) per (tile of up to 64 consecutive query tokens of one
+//   prefill kernel: one workgroup (8 waves) per (tile of up to 128 consecutive query tokens of one
 //                   request, head); keys and values of 64 positions at a time are staged in LDS.
 //   decode kernel:  one wave per (single-token query, kv head, split of the key range); operands go
 //                   from global memory straight into registers; the splits' partial results
@@ -522,6 +522,20 @@ __device__ __forceinline__ void prefill_tile(const bf16_t* __restrict__ q, long 
   }
 }
 
+// Workgroup b of n (n = H times the number of tiles, or of pairs of tiles): its tile (or pair) x and its head h.
+__device__ __forceinline__ void prefill_workgroup(int b, int n, int H, int KVH, int& x, int& h) {
+  const int n_x = n / H;
+  if (KVH % 8 == 0) {
+    const int xcd = b % 8, j = b / 8, G = H / KVH;
+    const int kvh = xcd + 8 * (j % (KVH / 8)), rest = j / (KVH / 8);  // rest counts (query head of the group, tile)
+    h = kvh * G + rest % G;
+    x = rest / G;
+  } else {
+    x = b % n_x;
+    h = b / n_x;
+  }
+}
+
 // The tiles come sorted by falling number of key blocks; with `pair`, workgroup x takes tile x and then tile n - 1 - x,
 // so that every workgroup has about the same work (a causal prompt's last tile reads many times more keys than its first).
 __global__ void __launch_bounds__(PF_THREADS)
@@ -536,17 +550,8 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
   // Workgroups go to the 8 XCDs in turn, each with an L2 of its own. A kv head's keys and values are read by every tile
   // of every query head that shares it: all of those run on one XCD (kv head % 8), so that the cache is fetched from
   // memory about once and not once per XCD (a 2,048-token prompt of 32 heads of 128: 34 MB a layer against 285 MB).
-  const int n_x = gridDim.x / H;  // tiles, or pairs of tiles
   int x, h;
-  if (KVH % 8 == 0) {
-    const int xcd = blockIdx.x % 8, j = blockIdx.x / 8, G = H / KVH;
-    const int kvh = xcd + 8 * (j % (KVH / 8)), rest = j / (KVH / 8);  // rest counts (query head of the group, tile)
-    h = kvh * G + rest % G;
-    x = rest / G;
-  } else {
-    x = blockIdx.x % n_x;
-    h = blockIdx.x / n_x;
-  }
+  prefill_workgroup(blockIdx.x, gridDim.x, H, KVH, x, h);
   const int first = x, second = n_tiles - 1 - x;
   prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * first],
                tiles[2 * first + 1], h, H, KVH, ps_shift, scale, window, softcap, score_bias, bias_len, Ks, Vs);
@@ -569,20 +574,20 @@ LEV_NAME(attn_prefill_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* _
 // range holds the token's own position takes them from k_new / v_new (rows of the projection's output) and
 // uses them in place of what the cache holds there; one wave copies them to dest[t] = page * PS + offset.
 #define DECODE_WG_WAVES 8
-__global__ void __launch_bounds__(64 * DECODE_WG_WAVES)
-LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
-                         bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
-                         const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
-                         const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
-                         const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
-                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
-                         int H, int KVH, int ps_shift, int splits, float scale, int window, int wg_merge, float softcap,
-                         const float* __restrict__ score_bias, int bias_len) {
+// One wave's work: single token number idx of the step, kv head kvh, key range z of `splits`.
+__device__ __forceinline__ void decode_wave(int idx, int kvh, int z, const bf16_t* __restrict__ q, long q_stride,
+                                            bf16_t* __restrict__ out, long o_stride, bf16_t* __restrict__ k_pages,
+                                            bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
+                                            const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
+                                            const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
+                                            const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
+                                            float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o, int H,
+                                            int KVH, int ps_shift, int splits, float scale, int window, int wg_merge, float softcap,
+                                            const float* __restrict__ score_bias, int bias_len) {
   const int PS = 1 << ps_shift, ps_mask = PS - 1;
   const float scale_log2 = scale * 1.4426950408889634f;
   const int lane = threadIdx.x & 63;
   const int fr = lane & 15, g = lane >> 4;
-  const int idx = blockIdx.x, kvh = blockIdx.y, z = wg_merge ? (int)(threadIdx.x >> 6) : (int)blockIdx.z;
   const int t = decode_tokens[idx];
   const int G = H / KVH;
   const int pos = positions[t];
@@ -799,6 +804,53 @@ LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __
   }
 }
 
+__global__ void __launch_bounds__(64 * DECODE_WG_WAVES)
+LEV_NAME(attn_decode_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                         bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
+                         const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
+                         const int* __restrict__ decode_tokens, const bf16_t* __restrict__ k_new,
+                         const bf16_t* __restrict__ v_new, long kv_stride, const int* __restrict__ dest,
+                         float* __restrict__ ws_m, float* __restrict__ ws_l, float* __restrict__ ws_o,
+                         int H, int KVH, int ps_shift, int splits, float scale, int window, int wg_merge, float softcap,
+                         const float* __restrict__ score_bias, int bias_len) {
+  decode_wave(blockIdx.x, blockIdx.y, wg_merge ? (int)(threadIdx.x >> 6) : (int)blockIdx.z, q, q_stride, out, o_stride, k_pages, v_pages,
+              positions, token_seq, block_tables, bt_stride, decode_tokens, k_new, v_new, kv_stride, dest, ws_m, ws_l, ws_o, H, KVH,
+              ps_shift, splits, scale, window, wg_merge, softcap, score_bias, bias_len);
+}
+
+// A step of prompt portions beside single tokens whose key ranges are not split: both kinds of work in one launch, so that
+// the single tokens' waves (bound by memory) fill the CUs that the portions' few workgroups (bound by latency) leave idle,
+// and the step has one kernel boundary fewer a layer. Workgroups below n_pf_wgs are the prefill kernel's, with its
+// numbering; each of the others is DECODE_WG_WAVES waves with a (single token, kv head) each, whose new keys and values
+// the KV-write kernel has written before.
+__global__ void __launch_bounds__(PF_THREADS)
+LEV_NAME(attn_mixed_hd)(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long o_stride,
+                        bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ positions,
+                        const int* __restrict__ token_seq, const int* __restrict__ block_tables, int bt_stride,
+                        const int* __restrict__ tiles, int n_tiles, int pair, int n_pf_wgs, const int* __restrict__ decode_tokens,
+                        int n_decode, int H, int KVH, int ps_shift, float scale, int window, float softcap,
+                        const float* __restrict__ score_bias, int bias_len) {
+  static_assert(PF_THREADS == 64 * DECODE_WG_WAVES, "one workgroup size for both kinds of work");
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][4][NCHUNK][16][8];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][VS_STRIDE];
+  if ((int)blockIdx.x < n_pf_wgs) {
+    int x, h;
+    prefill_workgroup(blockIdx.x, n_pf_wgs, H, KVH, x, h);
+    const int first = x, second = n_tiles - 1 - x;
+    prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * first],
+                 tiles[2 * first + 1], h, H, KVH, ps_shift, scale, window, softcap, score_bias, bias_len, Ks, Vs);
+    if (pair && second > first)
+      prefill_tile(q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride, tiles[2 * second],
+                   tiles[2 * second + 1], h, H, KVH, ps_shift, scale, window, softcap, score_bias, bias_len, Ks, Vs);
+    return;
+  }
+  const int item = ((int)blockIdx.x - n_pf_wgs) * DECODE_WG_WAVES + (int)(threadIdx.x >> 6);
+  if (item >= n_decode * KVH) return;
+  decode_wave(item / KVH, item % KVH, 0, q, q_stride, out, o_stride, k_pages, v_pages, positions, token_seq, block_tables, bt_stride,
+              decode_tokens, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, H, KVH, ps_shift, 1, scale, window, 0, softcap,
+              score_bias, bias_len);
+}
+
 // merge the splits of one (token, head): weights exp(m_z - max) per split, then a fixed-order sum
 __global__ void __launch_bounds__(64)
 LEV_NAME(attn_combine_hd)(bf16_t* __restrict__ out, long o_stride, const int* __restrict__ decode_tokens,
@@ -842,6 +894,17 @@ extern "C" int LEV_NAME(lev_attention_mfma_hd)(const void* q, long q_stride, voi
   int ps_shift = 0;
   while ((1 << ps_shift) < PS) ++ps_shift;
   if ((1 << ps_shift) != PS) return lev_fail("attention (matrix cores): page_size=%d must be a power of two", PS);
+  if (n_prefill_tiles > 0 && n_decode > 0 && splits == 1 && !k_new) {
+    const int pair = (long)n_prefill_tiles * H >= 512;
+    const int n_pf_wgs = (pair ? (n_prefill_tiles + 1) / 2 : n_prefill_tiles) * H;
+    const long items = (long)n_decode * KVH;
+    dim3 grid((unsigned)(n_pf_wgs + (items + DECODE_WG_WAVES - 1) / DECODE_WG_WAVES));
+    LEV_NAME(attn_mixed_hd)<<<grid, PF_THREADS, 0, stream>>>(
+        (const bf16_t*)q, q_stride, (bf16_t*)out, o_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, positions, token_seq, block_tables,
+        bt_stride, prefill_tiles, n_prefill_tiles, pair, n_pf_wgs, decode_tokens, n_decode, H, KVH, ps_shift, scale, window, softcap,
+        score_bias, bias_len);
+    return lev_check_launch("attention of a mixed step");
+  }
   if (n_prefill_tiles > 0) {
     // pairing halves the number of workgroups: only when every CU (256 of them) still gets one
     const int pair = (long)n_prefill_tiles * H >= 512;

@@ -694,6 +694,36 @@ def test_pools_of_more_than_two_to_the_31_elements(K, dtype):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("H,KVH,HD,PS,portions,singles", [
+    (25, 25, 64, 16, [(256, 256)], [450] * 64 + [1, 17, 64, 65] * 5),       # every key range whole: portions and single tokens in one launch
+    (32, 32, 128, 16, [(130, 300), (64, 64), (2, 2)], [640] * 61 + [1, 2, 700]),
+    (12, 4, 96, 32, [(30, 30), (20, 64)], [33, 64, 7] * 100),               # query heads that share keys
+    (8, 8, 128, 16, [(300, 300)], [900, 17]),                               # few single tokens: their key ranges are split, two launches
+])
+def test_a_mixed_step_s_attention_equals_its_two_halves(K, H, KVH, HD, PS, portions, singles):
+    """Prompt portions beside single tokens: where no single token's key range is split, one launch does both kinds of work.
+    Its output equals, bit for bit, that of the portions alone and of the single tokens alone (two steps over the same
+    cache), and the plain statement within rounding."""
+    dtype = torch.bfloat16
+    runs = list(portions) + [(1, n) for n in singles]
+    kv_lens = [k for _, k in runs]
+    n_pages = sum((k + PS - 1) // PS for k in kv_lens) + 3
+    bt, kp, vp, kd, vd, _, _ = _fill_cache(K, dtype, kv_lens, KVH, HD, PS, n_pages, seed=23)
+    T = sum(q for q, _ in runs)
+    n_pf = sum(q for q, _ in portions)
+    q = _rand(T, H * HD, dtype=dtype, seed=29).to(DEV)
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=1 / math.sqrt(HD) / 2, window=None)
+    got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q, got, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
+    halves = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
+    K.paged_attention(q[:n_pf], halves[:n_pf], kd, vd, make_meta(portions, DEV), block_tables=bt[:len(portions)].contiguous().to(DEV), **args)
+    K.paged_attention(q[n_pf:], halves[n_pf:], kd, vd, make_meta(runs[len(portions):], DEV), block_tables=bt[len(portions):].contiguous().to(DEV), **args)
+    assert torch.equal(got, halves)
+    want = torch.empty(T, H * HD, dtype=dtype)
+    EMU.paged_attention(q.cpu(), want, kp, vp, make_meta(runs, "cpu"), block_tables=bt, **args)
+    torch.testing.assert_close(got.cpu().float(), want.float(), rtol=2e-2, atol=2e-2)
+
+
 def test_paged_attention_random_cases(K):
     """Forty random cases in bfloat16: head sizes 16 .. 128, groups of query heads, page sizes, windows, prompt portions
     beside single tokens. Steps of single tokens also go through the kernel that takes the new key and value from
