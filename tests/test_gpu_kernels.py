@@ -396,27 +396,34 @@ def test_the_choice_between_the_two_kernels_for_a_few_rows_is_within_a_quarter_o
     that shares them and splits the sum over K. Here both are timed at ten shapes the estimate was not fitted to; the one
     it picks may be at most a quarter slower than the other."""
     gemm = K._unit("gemm_mfma")
-    report = []
+
+    def timed(M, N, K_, reps):
+        n_w = max(3, min(12, int(6e8 / (N * K_ * 2))))
+        weights = [_rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=i).to(DEV) for i in range(n_w)]
+        a = _rand(M, K_, dtype=torch.bfloat16, seed=1).to(DEV)
+        bias = _rand(N, seed=2).to(DEV)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        times = {}
+        for kind in (0, 1, 2):
+            K._check(gemm.lev_linear_mfma_force(kind))
+            K._ws_need.clear()  # the workspace a shape needs depends on the kernel that takes it
+            times[kind] = _time_products(lambda w: K.linear(a, w, bias, out, activation="gelu_new"), weights, reps=reps)
+        return times
+
+    def slower(t):
+        return t[0] > 1.25 * min(t[1], t[2])
+
     try:
-        for M, N, K_ in DISPATCH_SHAPES:
-            n_w = max(3, min(12, int(6e8 / (N * K_ * 2))))
-            weights = [_rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=i).to(DEV) for i in range(n_w)]
-            a = _rand(M, K_, dtype=torch.bfloat16, seed=1).to(DEV)
-            bias = _rand(N, seed=2).to(DEV)
-            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-            times = {}
-            for kind in (0, 1, 2):
-                K._check(gemm.lev_linear_mfma_force(kind))
-                K._ws_need.clear()  # the workspace a shape needs depends on the kernel that takes it
-                times[kind] = _time_products(lambda w: K.linear(a, w, bias, out, activation="gelu_new"), weights)
-            report.append((M, N, K_, times))
-            del weights
+        report = [(M, N, K_, timed(M, N, K_, 5)) for M, N, K_ in DISPATCH_SHAPES]
+        # a shape over the line is timed once more, three times as long, before it counts: a neighbour on the machine or a
+        # clock that has not settled moves a single measurement by several percent
+        report = [(M, N, K_, timed(M, N, K_, 15) if slower(t) else t) for M, N, K_, t in report]
     finally:
         K._check(gemm.lev_linear_mfma_force(0))
         K._ws_need.clear()
     lines = [f"M={M} N={N} K={K_}: chosen {t[0]:.1f} us, skinny {t[1]:.1f}, stream {t[2]:.1f}" for M, N, K_, t in report]
     print("\n".join(lines))
-    bad = [line for line, (_, _, _, t) in zip(lines, report) if t[0] > 1.25 * min(t[1], t[2])]
+    bad = [line for line, (_, _, _, t) in zip(lines, report) if slower(t)]
     assert not bad, "the estimate picks the slower kernel:\n" + "\n".join(bad)
 
 
@@ -428,20 +435,23 @@ def test_the_choice_between_own_kernels_and_the_vendor_library_is_within_a_quart
     """From 25 rows a rule by rows, shape and weight size sends a product to the vendor library or keeps it. Both are
     timed at ten shapes off the model sizes the rule was made from; the one it picks may be at most a quarter slower."""
     was = K.gemm_library
-    report = []
+
+    def timed(M, N, K_, reps):
+        n_w = max(3, min(12, int(6e8 / (N * K_ * 2))))
+        weights = [_rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=i).to(DEV) for i in range(n_w)]
+        a = _rand(M, K_, dtype=torch.bfloat16, seed=1).to(DEV)
+        bias = _rand(N, seed=2).to(DEV)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        times = {}
+        for lib in (True, False):
+            K.gemm_library = lib
+            times[lib] = _time_products(lambda w: K.linear(a, w, bias, out, activation="gelu_new"), weights, reps=reps)
+        return times
+
     try:
-        for M, N, K_ in LIBRARY_SHAPES:
-            n_w = max(3, min(12, int(6e8 / (N * K_ * 2))))
-            weights = [_rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=i).to(DEV) for i in range(n_w)]
-            a = _rand(M, K_, dtype=torch.bfloat16, seed=1).to(DEV)
-            bias = _rand(N, seed=2).to(DEV)
-            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-            times = {}
-            for lib in (True, False):
-                K.gemm_library = lib
-                times[lib] = _time_products(lambda w: K.linear(a, w, bias, out, activation="gelu_new"), weights)
-            report.append((M, N, K_, K.use_library(M, N, K_, 1), times))
-            del weights
+        report = [(M, N, K_, K.use_library(M, N, K_, 1), timed(M, N, K_, 5)) for M, N, K_ in LIBRARY_SHAPES]
+        # over the line: timed once more, three times as long, before it counts (see the test above)
+        report = [(M, N, K_, use, timed(M, N, K_, 15) if use and t[True] > 1.25 * t[False] else t) for M, N, K_, use, t in report]
     finally:
         K.gemm_library = was
     lines = [f"M={M} N={N} K={K_}: rule says {'library' if use else 'own'}; library (where the rule allows it) {t[True]:.1f} us, own {t[False]:.1f}"
