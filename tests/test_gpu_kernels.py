@@ -704,13 +704,14 @@ def test_pools_of_more_than_two_to_the_31_elements(K, dtype):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("H,KVH,HD,PS,portions,singles", [
-    (25, 25, 64, 16, [(256, 256)], [450] * 64 + [1, 17, 64, 65] * 5),       # every key range whole: portions and single tokens in one launch
-    (32, 32, 128, 16, [(130, 300), (64, 64), (2, 2)], [640] * 61 + [1, 2, 700]),
-    (12, 4, 96, 32, [(30, 30), (20, 64)], [33, 64, 7] * 100),               # query heads that share keys
-    (8, 8, 128, 16, [(300, 300)], [900, 17]),                               # few single tokens: their key ranges are split, two launches
+@pytest.mark.parametrize("H,KVH,HD,PS,portions,singles,window", [
+    (25, 25, 64, 16, [(256, 256)], [450] * 64 + [1, 17, 64, 65] * 5, None),  # every key range whole: portions and single tokens in one launch
+    (32, 32, 128, 16, [(130, 300), (64, 64), (2, 2)], [640] * 61 + [1, 2, 700], None),
+    (12, 4, 96, 32, [(30, 30), (20, 64)], [33, 64, 7] * 100, None),          # query heads that share keys
+    (16, 16, 64, 16, [(200, 333)], [300, 40, 129] * 30, 100),                # under a window
+    (8, 8, 128, 16, [(300, 300)], [900, 17], None),                          # few single tokens: their key ranges are split, two launches
 ])
-def test_a_mixed_step_s_attention_equals_its_two_halves(K, H, KVH, HD, PS, portions, singles):
+def test_a_mixed_step_s_attention_equals_its_two_halves(K, H, KVH, HD, PS, portions, singles, window):
     """Prompt portions beside single tokens: where no single token's key range is split, one launch does both kinds of work.
     Its output equals, bit for bit, that of the portions alone and of the single tokens alone (two steps over the same
     cache), and the plain statement within rounding."""
@@ -722,7 +723,7 @@ def test_a_mixed_step_s_attention_equals_its_two_halves(K, H, KVH, HD, PS, porti
     T = sum(q for q, _ in runs)
     n_pf = sum(q for q, _ in portions)
     q = _rand(T, H * HD, dtype=dtype, seed=29).to(DEV)
-    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=1 / math.sqrt(HD) / 2, window=None)
+    args = dict(n_heads=H, n_kv_heads=KVH, head_dim=HD, page_size=PS, scale=1 / math.sqrt(HD) / 2, window=window)
     got = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
     K.paged_attention(q, got, kd, vd, make_meta(runs, DEV), block_tables=bt.to(DEV), **args)
     halves = torch.full((T, H * HD), float("nan"), dtype=dtype, device=DEV)
