@@ -8,7 +8,8 @@
 //                 that do not fit the CUs): the weights are the traffic; `a` is shared through LDS by the 4 to 16 waves of a
 //                 workgroup, the weights go straight into MFMA operand registers, K is split over workgroups
 //                 and a second kernel adds the partial sums in a fixed order;
-//   skinny kernel (M <= 24, see use_skinny): a workgroup owns 16 output columns; its waves split K, load their part of w
+//   skinny kernel (M <= 24, and up to 64 rows of narrow layers, see use_skinny): a workgroup owns 16 output columns;
+//                 its waves split K, load their part of w
 //                 straight into MFMA operand registers (16x16x32), and their partial sums are added
 //                 through LDS in a fixed order.
 // No atomics anywhere: results are deterministic. K and lda must be multiples of 8 (16-byte operand loads);
@@ -331,7 +332,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Skinny kernel (M <= SKINNY_MAX_M: MT = 1 or 2 tiles of 16 rows). A workgroup owns NT = 1 to 3 units of 16 output columns; its WAVES
+// Skinny kernel (M <= SKINNY_MAX_M: MT = 1, 2 or 4 tiles of 16 rows). A workgroup owns NT = 1 to 3 units of 16 output columns; its WAVES
 // waves split K. A wave takes pairs of adjacent 32-wide k-steps (64 k = 128 bytes of a row), U pairs in flight:
 //   weights: lane (row l%16, k-group l/16) loads 16 bytes straight into the MFMA operand, two loads per pair;
 //   `a`:     read as WHOLE 128-byte lines - lane (row l/8, 16-byte chunk l%8), one instruction for rows 0..7 and one
@@ -343,7 +344,7 @@ static int launch_tile(const bf16_t* a, long lda, const bf16_t* w, const float* 
 // place of the k range, so that they do not all read the same part of `a` and the same residue of the weight
 // rows at the same time; the order of the sum depends on the column tile only, never on M or the batch.
 #define SKINNY_SLOTS 72  // 16-byte slots of one staged instruction: 8 rows x (8 chunks + 1 of padding)
-#define SKINNY_MAX_M 24  // with two row tiles; which of these row counts it takes: use_skinny()
+#define SKINNY_MAX_M 64  // with four row tiles; which of these row counts it takes: use_skinny()
 
 template <typename TO, int WAVES, int U, int ROT, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64)
@@ -351,8 +352,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
                    const float* residual, long ldr, TO* out, long ldo, int M, int N, int K, int act) {
   static_assert(NT >= 1 && NT <= WAVES, "wave j finishes column unit j");
   constexpr int AI = 2 * MT;  // `a` instructions per pair of k-steps: 8 rows each
+  // With more than two row tiles the staging area holds one tile at a time (the LDS executes a wave's instructions in
+  // order, so the next tile's writes cannot overtake this one's reads): 16 waves x 8 instructions would not fit the LDS.
+  constexpr bool ONE_TILE = MT > 2;
+  constexpr int SI = ONE_TILE ? 2 : AI;
   __shared__ f32x4 red[WAVES][NT][MT][64];
-  __shared__ u32x4 stage[WAVES][AI][SKINNY_SLOTS];
+  __shared__ u32x4 stage[WAVES][SI][SKINNY_SLOTS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * 16 * NT;
@@ -429,11 +434,18 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restr
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // LDS executes a wave's instructions in order: the area is reused pair after pair without a barrier
+      if (!ONE_TILE) {
 #pragma unroll
-      for (int i = 0; i < AI; ++i) my_stage[i * SKINNY_SLOTS + st_slot] = av[u][i];
+        for (int i = 0; i < AI; ++i) my_stage[i * SKINNY_SLOTS + st_slot] = av[u][i];
+      }
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const u32x4 a_lo = my_stage[2 * t * SKINNY_SLOTS + ld_slot], a_hi = my_stage[2 * t * SKINNY_SLOTS + ld_slot + 4];
+        if (ONE_TILE) {
+          my_stage[st_slot] = av[u][2 * t];
+          my_stage[SKINNY_SLOTS + st_slot] = av[u][2 * t + 1];
+        }
+        const int base = ONE_TILE ? 0 : 2 * t * SKINNY_SLOTS;
+        const u32x4 a_lo = my_stage[base + ld_slot], a_hi = my_stage[base + ld_slot + 4];
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(wv[u][j][0]), acc[j][t], 0, 0, 0);
@@ -501,8 +513,9 @@ static SkinnyShape skinny_shape(int M, int N) {
     if (tiles >= 512) return {4, 2, 1, 1};
     return {16, 1, 1, 1};
   }
-  // 17 .. SKINNY_MAX_M rows: two row tiles share every weight load
-  return tiles >= 512 ? SkinnyShape{4, 2, 2, 1} : SkinnyShape{16, 1, 2, 1};
+  // 17 .. 32 rows: two row tiles share every weight load; up to SKINNY_MAX_M: four
+  if (M <= 32) return tiles >= 512 ? SkinnyShape{4, 2, 2, 1} : SkinnyShape{16, 1, 2, 1};
+  return tiles >= 512 ? SkinnyShape{4, 2, 4, 1} : SkinnyShape{16, 1, 4, 1};
 }
 
 template <typename TO>
@@ -521,6 +534,8 @@ static void launch_skinny(const bf16_t* a, long lda, const bf16_t* w, const floa
   LEV_SKINNY(16, 1, 1, 1);
   LEV_SKINNY(4, 2, 2, 1);
   LEV_SKINNY(16, 1, 2, 1);
+  LEV_SKINNY(4, 2, 4, 1);
+  LEV_SKINNY(16, 1, 4, 1);
 #undef LEV_SKINNY
 }
 
@@ -847,6 +862,15 @@ extern "C" int lev_linear_mfma_force(int kind) {
 static bool use_skinny(int M, int N, int K) {
   if (M > SKINNY_MAX_M) return false;
   if (g_force_kernel) return g_force_kernel == 1;
+  if (M > 24) {
+    // 25 to 64 rows (two or four row tiles), microseconds skinny / stream, second kernel included, at 32 and 64 rows: where
+    // the skinny kernel's workgroups of 16 waves make one round of the CUs and the sum is no longer than the output is wide
+    // it stays ahead (2304 x 768: 5.2 / 7.6, 7.6 / 9.4; 4096 x 1024: 6.1 / 8.6, 8.9 / 10.4; 1600 x 1600: 6.5 / 8.4, 9.5 / 10.2;
+    // 4096 x 4096: 13.4 / 15.0 but 18.6 / 16.7), elsewhere not (4800 x 1600, 300 workgroups: 14.1 / 11.1, 20.4 / 13.4;
+    // 1024 x 4096: 11.4 / 9.3, 16.2 / 11.0; 12288 x 4096: 32.1 / 26.4, 42.4 / 28.7).
+    const int tiles = (N + 15) / 16;
+    return tiles <= 256 && K <= N && (M <= 32 || (long)N * K <= (1L << 23));
+  }
   return skinny_estimate(M, N, K) <= 1.3 * plan_stream(M, N, K).cost;
 }
 

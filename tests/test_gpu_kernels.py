@@ -167,6 +167,54 @@ def test_linear_bf16_random_shapes_strides_and_epilogues(K):
         assert err < tol, (M, K_, N, lda, act, with_res, with_bias, out.dtype, err)
 
 
+def test_linear_bf16_both_kernels_for_up_to_64_rows(K):
+    """Up to 64 rows either of two kernels may take a product (one whose workgroups each read all of the activations, with
+    one, two or four row tiles; one that shares them and splits the sum over K). Both are forced in turn over forty
+    random shapes with ragged widths, row strides above K and every epilogue, against the float64 statement; where both run
+    the same sum order is not required, only the tolerance."""
+    import random
+
+    rng = random.Random(19)
+    gemm = K._unit("gemm_mfma")
+    was = K.gemm_library
+    K.gemm_library = False
+    try:
+        for trial in range(40):
+            M = rng.choice([1, 7, 16, 17, 24, 25, 31, 32, 33, 40, 47, 48, 49, 63, 64])
+            K_ = 8 * rng.choice([1, 4, 8, 9, 25, 64, 96, 129, 200, 512])
+            N = rng.choice([1, 15, 16, 17, 100, 256, 257, 1000, 1600, 2304, 4097, 8200])
+            with_res, with_bias = rng.random() < 0.4, rng.random() < 0.7
+            act = "none" if with_res else rng.choice(["none", "relu", "gelu_new", "silu"])
+            lda = K_ + 8 * rng.choice([0, 0, 2])
+            a = _rand(M, lda, dtype=torch.bfloat16, seed=trial).to(DEV)[:, :K_]
+            w = _rand(N, K_, dtype=torch.bfloat16, scale=K_ ** -0.5, seed=100 + trial).to(DEV)
+            bias = _rand(N, seed=200 + trial).to(DEV) if with_bias else None
+            res = _rand(M, N, seed=300 + trial).to(DEV) if with_res else None
+            want = a.double() @ w.double().t()
+            if with_bias:
+                want = want + bias.double()
+            want = {"none": lambda x: x, "relu": torch.relu, "gelu_new": lambda x: torch.nn.functional.gelu(x, approximate="tanh"),
+                    "silu": torch.nn.functional.silu}[act](want)
+            if with_res:
+                want = want + res.double()
+            for kind in (1, 2):
+                K._check(gemm.lev_linear_mfma_force(kind))
+                K._ws_need.clear()
+                if with_res:
+                    out = res.clone()
+                    K.linear(a, w, bias, out, residual=out)
+                else:
+                    out = torch.full((M, N), float("nan"), device=DEV, dtype=rng.choice([torch.bfloat16, torch.float32]))
+                    K.linear(a, w, bias, out, activation=act)
+                tol = 2e-2 if out.dtype == torch.bfloat16 else 2e-3
+                err = float((out.double() - want).abs().max() / (want.abs().max() + 1e-6))
+                assert err < tol, (trial, kind, M, K_, N, lda, act, with_res, with_bias, out.dtype, err)
+    finally:
+        K._check(gemm.lev_linear_mfma_force(0))
+        K._ws_need.clear()
+        K.gemm_library = was
+
+
 @pytest.mark.parametrize("M,K_,N", [(64, 4096, 4096), (33, 4096, 3208), (100, 2048, 6151), (128, 8192, 1608), (48, 16384, 1000),
                                     (26, 4096, 12288), (64, 1024, 50257), (128, 4096, 16384), (32, 4096, 16384), (22, 4096, 8200)])
 def test_linear_bf16_large_weights_at_20_to_128_rows(K, M, K_, N):
@@ -388,13 +436,16 @@ def _time_products(fn, weights, reps=5):
 DISPATCH_SHAPES = [  # (M, N, K): widths between and beyond the three model sizes the estimates were fitted to
     (4, 3840, 1280), (16, 1280, 5120), (24, 7680, 2560), (8, 2560, 2560), (16, 20480, 5120), (24, 5120, 20480), (2, 768, 3072),
     (20, 10240, 2560), (12, 15360, 5120), (24, 2304, 768),
+    # 25 to 64 rows: narrow layers may stay with the first kernel
+    (32, 2048, 2048), (48, 3072, 1024), (64, 1280, 1280), (40, 2560, 2560), (64, 5120, 1280), (28, 1024, 4096), (56, 3840, 1280),
+    (32, 6144, 6144), (64, 2304, 768),
 ]
 
 
 def test_the_choice_between_the_two_kernels_for_a_few_rows_is_within_a_quarter_of_the_better_one(K):
     """Up to 24 rows an estimate decides between the kernel whose workgroups each read all of the activations and the one
-    that shares them and splits the sum over K. Here both are timed at ten shapes the estimate was not fitted to; the one
-    it picks may be at most a quarter slower than the other."""
+    that shares them and splits the sum over K, from 25 to 64 rows a rule by shape. Here both are timed at shapes that
+    neither was fitted to; the one that is picked may be at most a quarter slower than the other."""
     gemm = K._unit("gemm_mfma")
 
     def timed(M, N, K_, reps):
