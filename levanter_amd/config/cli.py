@@ -85,9 +85,38 @@ def from_dict(cls: Type[T], data: Dict[str, Any], path: str = "") -> T:
         raise ConfigError(f"{path or cls.__name__}: {e}") from None
 
 
+def describe_options(cls: Type, prefix: str = "") -> List[str]:
+    """One line per option of dataclass ``cls`` (sections as dotted names) with its type and default."""
+    lines: List[str] = []
+    hints = typing.get_type_hints(cls)
+    for f in dataclasses.fields(cls):
+        if not f.init:
+            continue
+        t = hints.get(f.name)
+        args = [a for a in typing.get_args(t) if a is not type(None)] if typing.get_origin(t) is typing.Union else []
+        target = t if dataclasses.is_dataclass(t) else next((a for a in args if dataclasses.is_dataclass(a)), None)
+        if target is not None:
+            lines += describe_options(target, prefix + f.name + ".")
+            continue
+        if f.default is not dataclasses.MISSING:
+            default = repr(f.default)
+        elif f.default_factory is not dataclasses.MISSING:  # type: ignore[misc]
+            default = repr(f.default_factory())  # type: ignore[misc]
+        else:
+            default = "required"
+        name = str(t).replace("typing.", "") if typing.get_origin(t) is not None else getattr(t, "__name__", str(t))
+        lines.append(f"  --{prefix}{f.name} ({name}; default {default})")
+    return lines
+
+
 def parse_config(cls: Type[T], argv: Optional[Sequence[str]] = None) -> T:
-    """``--config_path file.yaml`` (optional) plus overrides, into ``cls``."""
+    """``--config_path file.yaml`` (optional) plus overrides, into ``cls``. ``--help`` prints the options and exits."""
     argv = list(sys.argv[1:] if argv is None else argv)
+    if any(a in ("--help", "-h") for a in argv):
+        doc = (sys.modules[cls.__module__].__doc__ or "").strip()
+        print((doc + "\n\n" if doc else "") + "options (also as keys of the --config_path YAML file, sections nested):\n"
+              + "\n".join(describe_options(cls)))
+        raise SystemExit(0)
     over = parse_overrides(argv)
     base: Dict[str, Any] = {}
     path = over.pop("config_path", None) or over.pop("config", None)

@@ -30,3 +30,14 @@ def test_unknown_options_and_bad_values():
         main(SampleLmConfig())
     with pytest.raises(ConfigError, match="checkpoint_path"):
         main(SampleLmConfig(checkpoint_path="x"))
+
+
+def test_help_lists_every_option_with_its_default(capsys):
+    with pytest.raises(SystemExit) as e:
+        parse_config(SampleLmConfig, ["--help"])
+    assert e.value.code == 0
+    out = capsys.readouterr().out
+    for line in ("--hf_checkpoint (Optional[str]; default None)", "--engine.max_seqs (int; default 16)", "--engine.page_size (int; default 16)",
+                 "--trainer.mp (Optional[str]; default None)", "--max_new_tokens (int; default 192)", "--temperature (float; default 0.7)",
+                 "--n_rounds (int; default 4)", "--profile (bool; default False)"):
+        assert line in out, line
