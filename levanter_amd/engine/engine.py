@@ -72,6 +72,19 @@ class InferenceEngine:
         """The reference's constructor name (engine.py:705-731); the tokenizer is not needed: token ids in and out."""
         return cls(model, config or InferenceEngineConfig(), model.env)
 
+    @classmethod
+    def from_model(cls, model: DecoderLm, tokenizer=None, *, max_pages, max_seqs: int, page_size: int, max_pages_per_seq: int,
+                   compute_dtype=None, max_queued_tokens: int = 32, max_seqs_in_prefill: int = 16, max_prefill_size: Optional[int] = None):
+        """The reference's constructor from sizing arguments (engine.py:705-731). ``compute_dtype`` is the cache's dtype and
+        must be the dtype the model was built in (left out: that one)."""
+        built = {torch.bfloat16: "bfloat16", torch.float32: "float32"}[model.env.dtype]
+        name = built if compute_dtype is None else {torch.bfloat16: "bfloat16", torch.float32: "float32"}.get(compute_dtype, compute_dtype)
+        if name != built:
+            raise ValueError(f"from_model: the model was built in {built}, the cache cannot be {name}")
+        return cls.from_model_with_config(model, tokenizer, InferenceEngineConfig(
+            max_pages=max_pages, max_seqs=max_seqs, page_size=page_size, max_pages_per_seq=max_pages_per_seq, compute_dtype=name,
+            max_queued_tokens=max_queued_tokens, max_seqs_in_prefill=max_seqs_in_prefill, max_prefill_size=max_prefill_size))
+
     # ---- requests ---------------------------------------------------------------------------------
     def _validate(self, requests: Sequence[Request]) -> None:
         cfg = self.config

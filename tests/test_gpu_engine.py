@@ -150,6 +150,15 @@ def test_greedy_generation_through_the_entry_point(dtype):
         assert clear >= 40
     engine.cache.check_invariants()
     assert engine.cache.n_free_slots == 4
+    # the reference's constructors from a model that is already built (src/levanter/inference/engine.py:705-759): same tokens
+    from levanter_amd.engine import InferenceEngine
+
+    again = InferenceEngine.from_model(engine.model, None, max_pages=64, max_seqs=4, page_size=16, max_pages_per_seq=8,
+                                       compute_dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    assert again.generate([Request(prompt_tokens=p, request_id=i, max_new_tokens=16) for i, p in enumerate(prompts)]).tokens == res.tokens
+    with pytest.raises(ValueError, match="was built in"):
+        InferenceEngine.from_model(engine.model, None, max_pages=64, max_seqs=4, page_size=16, max_pages_per_seq=8,
+                                   compute_dtype="float32" if dtype == "bfloat16" else "bfloat16")
 
 
 def test_warm_up_leaves_the_engine_as_it_found_it():
