@@ -147,7 +147,7 @@ def test_greedy_generation_through_the_entry_point(dtype):
     else:
         # 47 of the 48 tokens have a margin that clear along the plain implementation's own path
         clear = sum(_check_greedy(w, TINY_A, p, out, P.bf16_rounding, margin=2e-2) for p, out in zip(prompts, res.tokens))
-        assert clear >= 40
+        assert clear >= 45
     engine.cache.check_invariants()
     assert engine.cache.n_free_slots == 4
     # the reference's constructors from a model that is already built (src/levanter/inference/engine.py:705-759): same tokens
@@ -325,7 +325,8 @@ def test_long_decoding_and_first_tokens(dtype):
     res = engine.generate([Request(prompt_tokens=[7], request_id=0, max_new_tokens=400)])
     out = res.tokens[0]
     assert len(out) == 255 and res.finish_reasons == ["length"]
-    assert _check_greedy(w, TINY_B, [7], out, rounding, margin) >= (250 if dtype == "float32" else 100)
+    # positions whose two best candidates are clearly apart (each of them is checked): 254 of 255 in bfloat16 as well
+    assert _check_greedy(w, TINY_B, [7], out, rounding, margin) >= (250 if dtype == "float32" else 245)
     # the first tokens: sequences of one, two and three tokens in one batch
     res = engine.generate([Request(prompt_tokens=[5], request_id=1, max_new_tokens=3),
                            Request(prompt_tokens=[9, 4], request_id=2, max_new_tokens=2),
