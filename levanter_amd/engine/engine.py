@@ -135,10 +135,18 @@ class InferenceEngine:
         settled afterwards: the request's row of the step launched ahead is ignored, and what that row wrote lies in
         pages that its request no longer owns and nobody reads."""
         t_step = time.perf_counter()
+        debug = logger.isEnabledFor(logging.DEBUG)
+        before = dict(self.stats) if debug else None
         try:
             return self._step()
         finally:
-            self.stats["step_s"] += time.perf_counter() - t_step
+            dt = time.perf_counter() - t_step
+            self.stats["step_s"] += dt
+            if debug:  # the reference logs every decode iteration's device and host time (engine.py:1146-1159)
+                wait = self.stats["wait_s"] - before["wait_s"]
+                logger.debug("step: %.3f ms (waiting for the GPU %.3f ms, host %.3f ms of which planning and launching %.3f ms), "
+                             "%d tokens in", 1e3 * dt, 1e3 * wait, 1e3 * (dt - wait), 1e3 * (self.stats["launch_s"] - before["launch_s"]),
+                             self.stats["tokens_in"] - before["tokens_in"])
 
     def _read(self, sample):
         t0 = time.perf_counter()
@@ -196,6 +204,7 @@ class InferenceEngine:
     def generate(self, requests: Sequence[Request]) -> GenerationResult:
         seqs = self.enqueue_requests(requests)
         t0 = time.perf_counter()
+        stats0 = dict(self.stats)
         idle_steps = 0
         while not all(s.done for s in seqs):
             # progress: a step was launched, a step launched earlier was committed, or a sequence ended (the planner
@@ -207,7 +216,9 @@ class InferenceEngine:
                 raise RuntimeError("the scheduler made no step twice in a row although requests are unfinished")
         dt = time.perf_counter() - t0
         total = sum(len(s.generated) for s in seqs)
-        logger.info("generated %d tokens in %.3fs (%.1f tok/s)", total, dt, total / max(dt, 1e-9))
+        wait = self.stats["wait_s"] - stats0["wait_s"]
+        logger.info("generated %d tokens in %.3fs (%.1f tok/s): %d steps, waiting for the GPU %.3fs, host %.3fs", total, dt,
+                    total / max(dt, 1e-9), self.stats["steps"] - stats0["steps"], wait, max(dt - wait, 0.0))
         want_lp = self.config.enable_logprobs and any(s.request.enable_logprobs for s in seqs)
         return GenerationResult(tokens=[list(s.generated) for s in seqs],
                                 logprobs=[list(s.logprobs) for s in seqs] if want_lp else None,
